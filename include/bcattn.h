@@ -1,0 +1,145 @@
+/*
+ * bcattn — block-causal (prefix-LM) attention for MI355X (gfx950), C ABI.
+ *
+ * This is the drop-in boundary for the one native interface the reference has on
+ * this path: the pybind module `opentau_flash_blockmask`
+ * (src/opentau/policies/flash_attn_cuda/_csrc/flash_blockmask.cu:1331-1334) with
+ *     flash_fwd(q,k,v,q_blk,k_blk,q_valid,k_valid,scale) -> [O, L]      (:1145-1208)
+ *     flash_bwd(dO,q,k,v,O,L,q_blk,k_blk,q_valid,k_valid,scale) -> [dQ,dK,dV] (:1210-1327)
+ * Here the same two operations, plus a KV-cached variant, are plain C functions
+ * over raw device pointers, element strides and an explicit HIP stream.  No
+ * torch types, no allocation: the caller owns every buffer (outputs and the
+ * workspace), nothing is retained after return, and every call is asynchronous
+ * with respect to the host on the stream it is given.
+ *
+ * Mask rule (flash_attn_cuda/__init__.py:27-28):
+ *     attend(i,j) = q_valid[i] && k_valid[j] && k_blk[j] <= q_blk[i]
+ * Block ids are int32 (cached / cross columns use INT32_MIN), valid flags are
+ * one byte per token.  No ordering of the ids is assumed.
+ * Head map: hk = h / (H / Hkv), H % Hkv == 0 (flash_blockmask.cu:157).
+ * Rows with no visible key (or q_valid == 0): O = 0, LSE = 0, no gradient
+ * (flash_blockmask.cu:240-244).
+ * LSE is fp32 (B,H,Sq) contiguous, natural log, scale already applied.
+ *
+ * Tensors are addressed as  ptr + b*stride_b + s*stride_s + h*stride_h + d  in
+ * ELEMENTS, the innermost (head_dim) axis contiguous; so (B,S,H,D), (B,H,S,D)
+ * and slices of a preallocated KV cache are all consumed without a copy.  Every
+ * base pointer must be 16-byte aligned and every stride a multiple of 8
+ * elements (bf16) or 4 elements (fp32).
+ *
+ * Supported: dtype BCATTN_BF16 with D in {64,128,256} (MFMA kernels) and
+ * BCATTN_F32 with D % 32 == 0, D <= 256 (exact fp32 kernels).  Anything else
+ * returns BCATTN_ERR_UNSUPPORTED with a message in bcattn_last_error().
+ */
+#ifndef BCATTN_H_
+#define BCATTN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BCATTN_ABI_VERSION 1
+
+enum bcattn_dtype { BCATTN_F32 = 0, BCATTN_BF16 = 1 };
+
+enum bcattn_status {
+  BCATTN_OK = 0,
+  BCATTN_ERR_INVALID = -1,     /* null pointer, bad shape, misaligned pointer or stride */
+  BCATTN_ERR_UNSUPPORTED = -2, /* dtype / head_dim the kernels do not cover */
+  BCATTN_ERR_WORKSPACE = -3,   /* workspace missing or too small */
+  BCATTN_ERR_LAUNCH = -4       /* the HIP runtime refused a launch */
+};
+
+/* One 4-D operand: element strides of the batch, sequence and head axes. */
+typedef struct bcattn_tensor {
+  void *ptr;
+  int64_t stride_b, stride_s, stride_h;
+} bcattn_tensor;
+
+/*
+ * Forward.  Keys/values come in up to two segments that are logically
+ * concatenated along the sequence axis: segment 0 (k, v: Sk0 rows — e.g. the
+ * cached VLM prefix) then segment 1 (k1, v1: Sk1 rows — e.g. this step's own
+ * block).  This replaces the torch.cat in
+ * src/opentau/policies/pi05/paligemma_with_expert.py:747-748.  Plain
+ * self-attention passes Sk1 = 0 and null k1/v1.  k_blk / k_valid cover the
+ * concatenation: (B, Sk0+Sk1) contiguous.
+ */
+typedef struct bcattn_fwd_params {
+  bcattn_tensor q;       /* (B,Sq,H,D)   in */
+  bcattn_tensor k, v;    /* (B,Sk0,Hkv,D) in */
+  bcattn_tensor k1, v1;  /* (B,Sk1,Hkv,D) in, may be null when Sk1 == 0 */
+  bcattn_tensor o;       /* (B,Sq,H,D)   out */
+  float *lse;            /* (B,H,Sq) out, may be null */
+  const int32_t *q_blk;  /* (B,Sq) */
+  const int32_t *k_blk;  /* (B,Sk0+Sk1) */
+  const uint8_t *q_valid;
+  const uint8_t *k_valid;
+  int32_t B, Sq, Sk0, Sk1, H, Hkv, D;
+  int32_t dtype; /* enum bcattn_dtype */
+  float scale;
+  /*
+   * Nonzero: `workspace` already holds the key-tile summary this call would
+   * compute (same k_blk/k_valid, same B and Sk) — e.g. from the previous layer,
+   * whose mask is identical — and the summary pass is skipped.
+   */
+  int32_t summary_ready;
+  void *workspace;
+  size_t workspace_bytes;
+} bcattn_fwd_params;
+
+/*
+ * Backward.  dq/dk/dv are fully overwritten (no accumulate).  Deterministic:
+ * no atomics; two calls on the same inputs give bit-identical gradients.
+ */
+typedef struct bcattn_bwd_params {
+  bcattn_tensor q, k, v, o, d_o; /* in  */
+  bcattn_tensor dq, dk, dv;      /* out */
+  const float *lse;              /* (B,H,Sq) from the forward */
+  const int32_t *q_blk, *k_blk;
+  const uint8_t *q_valid, *k_valid;
+  int32_t B, Sq, Sk, H, Hkv, D;
+  int32_t dtype;
+  float scale;
+  void *workspace;
+  size_t workspace_bytes;
+} bcattn_bwd_params;
+
+/* Replaces nothing in the reference; version handshake for the binding. */
+int bcattn_abi_version(void);
+
+/* Thread-local message for the last non-OK status returned on this thread.
+ * Stands in for the TORCH_CHECK text of flash_blockmask.cu:1137-1143. */
+const char *bcattn_last_error(void);
+
+/* Bytes of device workspace the call needs (0 is possible).  The reference
+ * allocates its own scratch with at::empty (flash_blockmask.cu:1226, :1295-1296);
+ * here the caller allocates it. */
+size_t bcattn_fwd_workspace_bytes(const bcattn_fwd_params *p);
+size_t bcattn_fwd_kvcache_workspace_bytes(const bcattn_fwd_params *p);
+size_t bcattn_bwd_workspace_bytes(const bcattn_bwd_params *p);
+
+/* Replaces flash_fwd (flash_blockmask.cu:1145-1208). `stream` is a hipStream_t. */
+int bcattn_fwd(const bcattn_fwd_params *p, void *stream);
+
+/*
+ * KV-cached suffix forward: few query rows (Sq*H/Hkv small, e.g. the 50 action
+ * tokens of a flow-matching denoise step) against a long cached segment 0 plus
+ * their own segment 1.  Same result as bcattn_fwd on the same params; the work
+ * is split over the key axis so that a handful of (batch, kv-head) problems
+ * still fill the GPU.  Replaces the cat + attention of
+ * paligemma_with_expert.py:742-768 inside the loop of
+ * src/opentau/policies/pi05/modeling_pi05.py:2015-2046.
+ */
+int bcattn_fwd_kvcache(const bcattn_fwd_params *p, void *stream);
+
+/* Replaces flash_bwd (flash_blockmask.cu:1210-1327). */
+int bcattn_bwd(const bcattn_bwd_params *p, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BCATTN_H_ */

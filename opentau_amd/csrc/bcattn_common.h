@@ -1,0 +1,191 @@
+// Shared device helpers for the gfx950 block-causal attention kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "bcattn.h"
+
+namespace bcattn {
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+constexpr int kIntMax = 0x7fffffff;
+constexpr int kIntMin = (-0x7fffffff - 1);
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// Key tiles of the summary pass are this many keys wide.
+constexpr int kSumTile = 64;
+
+// Per key tile: x = min block id over valid keys (INT_MAX when none),
+// y = max block id over valid keys (INT_MIN when none), z = 1 when every key of
+// the tile is in range and valid, w = number of valid keys.
+typedef i32x4 tile_summary_t;
+
+// D(32x32 fp32) += A(32x16 bf16) * B(16x32 bf16).
+// Lane l supplies A[row l%32][k 8*(l/32)..+7] and B[k 8*(l/32)..+7][col l%32];
+// it receives D[row 8*(r/4) + 4*(l/32) + r%4][col l%32] in register r.
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+// Row of the 32x32 accumulator held in register r by a lane of half hh.
+__device__ __forceinline__ constexpr int acc_row(int r, int hh) {
+  return 8 * (r >> 2) + 4 * hh + (r & 3);
+}
+
+// Value held by the lane 32 away (lane ^ 32).
+__device__ __forceinline__ float swap32(float x) {
+  return __shfl_xor(x, 32, 64);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ int wave_max_i(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ int wave_min_i(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ int wave_sum_i(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_sum_f(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// Eight fp32 -> eight bf16 (round to nearest even), one MFMA operand.
+__device__ __forceinline__ bf16x8 pack8(float a0, float a1, float a2, float a3, float a4, float a5,
+                                        float a6, float a7) {
+  bf16x8 r;
+  r[0] = (bf16_t)a0;
+  r[1] = (bf16_t)a1;
+  r[2] = (bf16_t)a2;
+  r[3] = (bf16_t)a3;
+  r[4] = (bf16_t)a4;
+  r[5] = (bf16_t)a5;
+  r[6] = (bf16_t)a6;
+  r[7] = (bf16_t)a7;
+  return r;
+}
+
+// ---------------------------------------------------------------------------
+// LDS layouts.
+//
+// "Row" tiles (keys or queries as rows, head_dim contiguous) are padded by 8
+// elements per row so that a 16-byte read by 16 consecutive rows touches every
+// bank once.
+//
+// "Transposed" tiles hold X^T: one row per head_dim index, 64 sequence
+// positions per row (128 bytes), so that an MFMA operand whose contraction
+// index is the sequence position is one 16-byte read.  Inside a row the 64
+// positions are permuted so that the operand built from a 32x32 accumulator
+// (which gives a lane rows 4*hh..4*hh+3 and 8+4*hh..8+4*hh+3 of each group of 16)
+// meets the matching positions, and 16-byte chunks are XOR-swizzled by the row
+// to keep both the transposing writes and the reads spread over the banks.
+// ---------------------------------------------------------------------------
+template <int D>
+struct RowTile {
+  static constexpr int kPitch = D + 8;
+};
+
+__device__ __forceinline__ int tr_swz(int d) { return ((d >> 1) ^ (d >> 4)) & 7; }
+
+// Element offset, inside a transposed 64-wide row d, of the 16-byte chunk that
+// holds contraction step kk (0..3), lane half hh.
+__device__ __forceinline__ int tr_read_off(int d, int kk, int hh) {
+  return d * 64 + 8 * (((2 * kk + hh)) ^ tr_swz(d));
+}
+
+// Element offset, inside transposed row d, of the 4 consecutive positions
+// 4*kg..4*kg+3 (kg = 0..15) of the 64-wide tile.
+__device__ __forceinline__ int tr_write_off(int d, int kg) {
+  const int chunk = 2 * (kg >> 2) + (kg & 1);
+  const int half = (kg & 3) >> 1;
+  return d * 64 + 8 * (chunk ^ tr_swz(d)) + 4 * half;
+}
+
+// Store a 4(positions) x 8(head_dim) block, given as four 8-wide rows, into the
+// transposed tile: eight 8-byte writes.
+__device__ __forceinline__ void tr_store_4x8(bf16_t *tile, int d0, int kg, bf16x8 r0, bf16x8 r1,
+                                             bf16x8 r2, bf16x8 r3) {
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    bf16x4 w;
+    w[0] = r0[e];
+    w[1] = r1[e];
+    w[2] = r2[e];
+    w[3] = r3[e];
+    *reinterpret_cast<bf16x4 *>(tile + tr_write_off(d0 + e, kg)) = w;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Kernel argument blocks (device pointers already offset to element 0).
+// ---------------------------------------------------------------------------
+struct TensorArg {
+  const void *ptr;
+  int64_t sb, ss, sh;
+};
+
+struct FwdArgs {
+  TensorArg q, k0, v0, k1, v1;
+  void *o;
+  int64_t o_sb, o_ss, o_sh;
+  float *lse;
+  const int32_t *q_blk, *k_blk;
+  const uint8_t *q_valid, *k_valid;
+  const tile_summary_t *ksum;  // (B, ceil(Sk/64))
+  int B, Sq, Sk0, Sk, H, Hkv, G;
+  float scale;
+};
+
+struct BwdArgs {
+  TensorArg q, k, v, o, d_o;
+  void *dq, *dk, *dv;
+  int64_t dq_sb, dq_ss, dq_sh, dk_sb, dk_ss, dk_sh, dv_sb, dv_ss, dv_sh;
+  const float *lse;
+  float *delta;  // (B,H,Sq)
+  const int32_t *q_blk, *k_blk;
+  const uint8_t *q_valid, *k_valid;
+  const tile_summary_t *ksum;  // (B, ceil(Sk/64))
+  const tile_summary_t *qsum;  // (B, ceil(Sq/64))
+  int B, Sq, Sk, H, Hkv, G;
+  float scale;
+};
+
+// kernel launchers, one translation unit each
+int launch_summary(const int32_t *blk, const uint8_t *valid, int B, int S, tile_summary_t *out,
+                   hipStream_t st);
+int launch_fwd_bf16(const FwdArgs &a, int D, hipStream_t st);
+int launch_fwd_f32(const FwdArgs &a, int D, hipStream_t st);
+int launch_bwd_bf16(const BwdArgs &a, int D, hipStream_t st);
+int launch_bwd_f32(const BwdArgs &a, int D, hipStream_t st);
+
+struct SplitArgs {
+  float *part_o;   // (B, Hkv, nsplit, R, D) fp32, R = G*Sq
+  float *part_ml;  // (B, Hkv, nsplit, R, 2) fp32: running max (raw scores), sum
+  int nsplit;
+};
+int launch_fwd_kvcache_bf16(const FwdArgs &a, const SplitArgs &s, int D, hipStream_t st);
+size_t kvcache_workspace_bytes(int B, int Sq, int Sk, int H, int Hkv, int D, int *nsplit_out);
+
+}  // namespace bcattn

@@ -1,0 +1,273 @@
+// Block-causal attention forward, bf16 in / fp32 accumulate, gfx950 MFMA.
+//
+// One workgroup = 4 waves = 128 "packed" query rows of one (batch, kv head):
+// packed row r = g*Sq + i runs over the G = H/Hkv query heads that share the kv
+// head, so MQA/GQA heads reuse the same K/V tile in LDS.  A wave owns 32 rows;
+// lane l owns row l%32 (its running max / sum / block id live in scalars of the
+// lane) and the two lane halves split the contraction index.
+//
+// Scores are computed transposed, S^T = K Q^T (keys x queries), so that the
+// softmax reduction over keys is in-lane plus one exchange with lane^32, and so
+// that the 32x32 accumulator of S^T is already laid out as the B operand of
+// O^T = V^T P^T.  K tiles sit in LDS as rows, V tiles transposed.
+#include "bcattn_common.h"
+
+namespace bcattn {
+
+template <int D>
+__global__ __launch_bounds__(256) void fwd_bf16_kernel(const FwdArgs a) {
+  constexpr int BN = 64;
+  constexpr int KP = RowTile<D>::kPitch;
+  constexpr int DK = D / 16;   // contraction steps of K Q^T
+  constexpr int DB = D / 32;   // 32-row blocks of O^T
+  constexpr int CPR = D / 8;   // 16-byte chunks per row
+  constexpr int KCH = (BN * CPR) / 256;
+  constexpr int VUNITS = 16 * CPR;  // 4x8 transposition units per V tile
+  constexpr int VUN = (VUNITS + 255) / 256;
+
+  __shared__ __align__(16) bf16_t Ks[BN * KP];
+  __shared__ __align__(16) bf16_t Vt[D * BN];
+  __shared__ __align__(16) int kb_s[BN];
+  __shared__ int red_s[8];
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int n = lane & 31, hh = lane >> 5;
+
+  const int R = a.G * a.Sq;
+  const int ntile_r = (R + 127) / 128;
+  int bid = blockIdx.x;
+  const int tile = bid % ntile_r;
+  bid /= ntile_r;
+  const int hk = bid % a.Hkv;
+  const int b = bid / a.Hkv;
+
+  // ---- this lane's query row ------------------------------------------------
+  const int r = tile * 128 + wave * 32 + n;
+  const bool rowok = r < R;
+  const int rr = rowok ? r : R - 1;
+  const int g = rr / a.Sq;
+  const int i = rr - g * a.Sq;
+  const int h = hk * a.G + g;
+  const bool qv = rowok && a.q_valid[(int64_t)b * a.Sq + i] != 0;
+  const int qb = qv ? a.q_blk[(int64_t)b * a.Sq + i] : kIntMin;
+
+  const bf16_t *qptr =
+      reinterpret_cast<const bf16_t *>(a.q.ptr) + b * a.q.sb + (int64_t)i * a.q.ss + h * a.q.sh;
+  bf16x8 qf[DK];
+#pragma unroll
+  for (int ks = 0; ks < DK; ++ks)
+    qf[ks] = *reinterpret_cast<const bf16x8 *>(qptr + 16 * ks + 8 * hh);
+
+  // ---- block-id range of the wave and of the workgroup ------------------------
+  const int qmax_w = wave_max_i(qv ? qb : kIntMin);
+  const int qmin_w = wave_min_i(qv ? qb : kIntMax);
+  const int any_w = wave_max_i(qv ? 1 : 0);
+  if (lane == 0) {
+    red_s[wave] = qmax_w;
+    red_s[4 + wave] = any_w;
+  }
+  __syncthreads();
+  const int qmax_g = max(max(red_s[0], red_s[1]), max(red_s[2], red_s[3]));
+  const int any_g = red_s[4] | red_s[5] | red_s[6] | red_s[7];
+
+  const int Sk = a.Sk;
+  const int nt = any_g ? (Sk + BN - 1) / BN : 0;
+  const tile_summary_t *ksum = a.ksum + (int64_t)b * ((Sk + BN - 1) / BN);
+
+  const bf16_t *k0b = reinterpret_cast<const bf16_t *>(a.k0.ptr) + b * a.k0.sb + hk * a.k0.sh;
+  const bf16_t *v0b = reinterpret_cast<const bf16_t *>(a.v0.ptr) + b * a.v0.sb + hk * a.v0.sh;
+  const bf16_t *k1b = reinterpret_cast<const bf16_t *>(a.k1.ptr) + b * a.k1.sb + hk * a.k1.sh;
+  const bf16_t *v1b = reinterpret_cast<const bf16_t *>(a.v1.ptr) + b * a.v1.sb + hk * a.v1.sh;
+  const int Sk0 = a.Sk0;
+
+  bf16x8 kreg[KCH];
+  bf16x8 vreg[VUN][4];
+  int kbreg = kIntMax;
+
+  auto next_needed = [&](int t) {
+    while (t < nt && ksum[t].x > qmax_g) ++t;
+    return t;
+  };
+
+  auto prefetch = [&](int t) {
+    const int j0 = t * BN;
+#pragma unroll
+    for (int it = 0; it < KCH; ++it) {
+      const int c = tid + 256 * it;
+      const int row = c / CPR, col = c % CPR;
+      const int j = j0 + row;
+      bf16x8 val = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (j < Sk) {
+        const bf16_t *p = (j < Sk0) ? k0b + (int64_t)j * a.k0.ss : k1b + (int64_t)(j - Sk0) * a.k1.ss;
+        val = *reinterpret_cast<const bf16x8 *>(p + col * 8);
+      }
+      kreg[it] = val;
+    }
+#pragma unroll
+    for (int it = 0; it < VUN; ++it) {
+      const int u = tid + 256 * it;
+      const int dch = u % CPR, kg = u / CPR;
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const int j = j0 + 4 * kg + x;
+        bf16x8 val = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (u < VUNITS && j < Sk) {
+          const bf16_t *p =
+              (j < Sk0) ? v0b + (int64_t)j * a.v0.ss : v1b + (int64_t)(j - Sk0) * a.v1.ss;
+          val = *reinterpret_cast<const bf16x8 *>(p + dch * 8);
+        }
+        vreg[it][x] = val;
+      }
+    }
+    if (tid < BN) {
+      const int j = j0 + tid;
+      kbreg = kIntMax;
+      if (j < Sk && a.k_valid[(int64_t)b * Sk + j]) kbreg = a.k_blk[(int64_t)b * Sk + j];
+    }
+  };
+
+  auto stage = [&]() {
+#pragma unroll
+    for (int it = 0; it < KCH; ++it) {
+      const int c = tid + 256 * it;
+      const int row = c / CPR, col = c % CPR;
+      *reinterpret_cast<bf16x8 *>(Ks + row * KP + col * 8) = kreg[it];
+    }
+#pragma unroll
+    for (int it = 0; it < VUN; ++it) {
+      const int u = tid + 256 * it;
+      const int dch = u % CPR, kg = u / CPR;
+      if (u < VUNITS) tr_store_4x8(Vt, 8 * dch, kg, vreg[it][0], vreg[it][1], vreg[it][2], vreg[it][3]);
+    }
+    if (tid < BN) kb_s[tid] = kbreg;
+  };
+
+  // ---- running state ---------------------------------------------------------
+  f32x16 o[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int x = 0; x < 16; ++x) o[db][x] = 0.f;
+  float m = -INFINITY;  // running max of the raw (unscaled) scores
+  float l = 0.f;        // this lane half's share of the running sum
+  const float c = a.scale * kLog2e;
+
+  int t = next_needed(0);
+  if (t < nt) prefetch(t);
+  while (t < nt) {
+    stage();
+    __syncthreads();
+    const tile_summary_t sm = ksum[t];
+    const int tn = next_needed(t + 1);
+    if (tn < nt) prefetch(tn);
+
+    if (sm.x <= qmax_w) {  // wave-uniform: some row of this wave sees some key of the tile
+      f32x16 s[2];
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) {
+#pragma unroll
+        for (int x = 0; x < 16; ++x) s[mb][x] = 0.f;
+        const bf16_t *kp = Ks + (32 * mb + n) * KP + 8 * hh;
+#pragma unroll
+        for (int ks = 0; ks < DK; ++ks) {
+          const bf16x8 ka = *reinterpret_cast<const bf16x8 *>(kp + 16 * ks);
+          s[mb] = mfma32(ka, qf[ks], s[mb]);
+        }
+      }
+      const bool needmask = !(sm.z != 0 && sm.y <= qmin_w);
+      if (needmask) {
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+          for (int r4 = 0; r4 < 4; ++r4) {
+            const i32x4 kb4 = *reinterpret_cast<const i32x4 *>(kb_s + 32 * mb + 8 * r4 + 4 * hh);
+#pragma unroll
+            for (int x = 0; x < 4; ++x)
+              if (kb4[x] > qb) s[mb][4 * r4 + x] = -INFINITY;
+          }
+      }
+      float mloc = s[0][0];
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int x = 0; x < 16; ++x) mloc = fmaxf(mloc, s[mb][x]);
+      mloc = fmaxf(mloc, swap32(mloc));
+      const float mnew = fmaxf(m, mloc);
+      const float moff = (mnew == -INFINITY) ? 0.f : mnew * c;
+      if (__any(mnew > m)) {
+        const float corr = fast_exp2(m * c - moff);
+        l *= corr;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int x = 0; x < 16; ++x) o[db][x] *= corr;
+      }
+      m = mnew;
+      bf16x8 pb[4];
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) {
+        float p[16];
+#pragma unroll
+        for (int x = 0; x < 16; ++x) {
+          p[x] = fast_exp2(s[mb][x] * c - moff);
+          l += p[x];
+        }
+        pb[2 * mb] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
+        pb[2 * mb + 1] = pack8(p[8], p[9], p[10], p[11], p[12], p[13], p[14], p[15]);
+      }
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const int d = 32 * db + n;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          const bf16x8 va = *reinterpret_cast<const bf16x8 *>(Vt + tr_read_off(d, kk, hh));
+          o[db] = mfma32(va, pb[kk], o[db]);
+        }
+      }
+    }
+    __syncthreads();
+    t = tn;
+  }
+
+  // ---- epilogue ----------------------------------------------------------------
+  l += swap32(l);
+  const bool has = qv && l > 0.f;
+  const float inv = has ? 1.f / l : 0.f;
+  if (rowok) {
+    if (a.lse != nullptr && hh == 0)
+      a.lse[((int64_t)b * a.H + h) * a.Sq + i] = has ? m * a.scale + __logf(l) : 0.f;
+    bf16_t *optr = reinterpret_cast<bf16_t *>(a.o) + b * a.o_sb + (int64_t)i * a.o_ss + h * a.o_sh;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        bf16x4 w;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) w[x] = (bf16_t)(o[db][4 * r4 + x] * inv);
+        *reinterpret_cast<bf16x4 *>(optr + 32 * db + 8 * r4 + 4 * hh) = w;
+      }
+  }
+}
+
+int launch_fwd_bf16(const FwdArgs &a, int D, hipStream_t st) {
+  const int R = a.G * a.Sq;
+  const int ntile_r = (R + 127) / 128;
+  const dim3 grid((unsigned)(ntile_r * a.Hkv * a.B)), block(256);
+  switch (D) {
+    case 64:
+      hipLaunchKernelGGL(fwd_bf16_kernel<64>, grid, block, 0, st, a);
+      break;
+    case 128:
+      hipLaunchKernelGGL(fwd_bf16_kernel<128>, grid, block, 0, st, a);
+      break;
+    case 256:
+      hipLaunchKernelGGL(fwd_bf16_kernel<256>, grid, block, 0, st, a);
+      break;
+    default:
+      return BCATTN_ERR_UNSUPPORTED;
+  }
+  return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
+}
+
+}  // namespace bcattn

@@ -1,0 +1,386 @@
+"""Block-causal flash attention for MI355X with the mask rebuilt in-kernel.
+
+Same public surface as the reference's op-level package
+(``src/opentau/policies/flash_attn_cuda/__init__.py:44-50``):
+
+  - :func:`make_att_block_ids` -- ``(q_blk, k_blk, q_valid, k_valid)`` from the
+    ``pad_masks`` / ``att_masks`` the policies already build.
+  - :func:`flash_attn_blockmask` -- autograd-aware attention on that compact form.
+  - :func:`is_available`, :func:`load_error`, :data:`INT_BLK_MIN`.
+
+plus :func:`flash_attn_blockmask_kvcache`, which takes the cached prefix K/V and
+this step's K/V as two segments instead of a ``torch.cat`` of both
+(``src/opentau/policies/pi05/paligemma_with_expert.py:747-748``).
+
+``attend(i, j) == q_valid[i] & k_valid[j] & (k_blk[j] <= q_blk[i])``; the dense
+``(B, Sq, Sk)`` mask is never built.  The kernels are reached through the C ABI
+of ``include/bcattn.h``; there is no fallback when they are unavailable.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from . import _loader
+from ._loader import is_available, load_error
+
+__all__ = [
+    "INT_BLK_MIN",
+    "flash_attn_blockmask",
+    "flash_attn_blockmask_kvcache",
+    "is_available",
+    "load_error",
+    "make_att_block_ids",
+]
+
+# Block id of cross-attention / cached columns: <= every cumsum id, so those
+# columns are visible to every query (subject to padding).
+INT_BLK_MIN = -(2**31)
+
+
+def make_att_block_ids(
+    pad_masks: torch.Tensor,
+    att_masks: torch.Tensor,
+    n_cross_att_tokens: int | None = None,
+    cross_att_pad_masks: torch.Tensor | None = None,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Compact form of the block-causal mask.
+
+    Same contract as the reference's ``make_att_block_ids``
+    (``src/opentau/policies/flash_attn_cuda/__init__.py:58-109``).
+
+    Args:
+        pad_masks: bool ``(B, N)``, True where the token is real.
+        att_masks: int/bool/float ``(B, N)``, 1 opens a new block, 0 continues it.
+        n_cross_att_tokens: prepend that many always-visible key columns.
+        cross_att_pad_masks: bool ``(B, n_cross_att_tokens)``; required with it.
+
+    Returns:
+        ``(q_blk int32 (B,N), k_blk int32 (B,[n_cross+]N), q_valid bool, k_valid bool)``.
+    """
+    if att_masks.ndim != 2:
+        raise ValueError(f"att_masks must be 2D, got {att_masks.ndim}")
+    if pad_masks.ndim != 2:
+        raise ValueError(f"pad_masks must be 2D, got {pad_masks.ndim}")
+    blk = torch.cumsum(att_masks.to(torch.int32), dim=1).to(torch.int32)
+    valid = pad_masks.to(torch.bool)
+    if n_cross_att_tokens is None:
+        return blk, blk, valid, valid
+    assert cross_att_pad_masks is not None, (
+        "cross_att_pad_masks must be provided if n_cross_att_tokens is provided"
+    )
+    assert cross_att_pad_masks.shape == (att_masks.size(0), n_cross_att_tokens), (
+        "cross_att_pad_masks must have shape (batch_size, n_cross_att_tokens)"
+    )
+    cross = blk.new_full((att_masks.size(0), n_cross_att_tokens), INT_BLK_MIN)
+    k_blk = torch.cat([cross, blk], dim=1)
+    k_valid = torch.cat([cross_att_pad_masks.to(torch.bool), valid], dim=1)
+    return blk, k_blk, valid, k_valid
+
+
+# --------------------------------------------------------------------------- #
+# raw calls through the C ABI
+# --------------------------------------------------------------------------- #
+_DTYPES = {torch.float32: (_loader.DTYPE_F32, 4), torch.bfloat16: (_loader.DTYPE_BF16, 8)}
+
+
+def _operand(t: torch.Tensor, vec: int) -> torch.Tensor:
+    """A view the kernels can address: unit innermost stride, aligned base and strides."""
+    if (
+        t.stride(3) != 1
+        or t.data_ptr() % 16
+        or t.stride(0) % vec
+        or t.stride(1) % vec
+        or t.stride(2) % vec
+    ):
+        return t.contiguous()
+    return t
+
+
+def _t4(t: torch.Tensor | None) -> _loader.Tensor4:
+    if t is None:
+        return _loader.Tensor4(None, 0, 0, 0)
+    return _loader.Tensor4(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
+
+
+def _ids(blk: torch.Tensor, valid: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    return blk.to(torch.int32).contiguous(), valid.to(torch.bool).contiguous()
+
+
+def _check(rc: int, lib) -> None:
+    if rc != _loader.OK:
+        raise RuntimeError(f"bcattn: {lib.bcattn_last_error().decode()} (status {rc})")
+
+
+def _stream(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _check_inputs(q, k, v):
+    if not q.is_cuda:
+        raise RuntimeError("flash_hip attention needs tensors on a HIP device; there is no CPU fallback")
+    if q.dtype not in _DTYPES:
+        raise RuntimeError(f"flash_hip attention supports float32 and bfloat16, got {q.dtype}")
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise RuntimeError("q, k and v must share one dtype")
+    if q.ndim != 4 or k.ndim != 4 or v.ndim != 4:
+        raise RuntimeError("q, k, v must be (B, S, H, D)")
+
+
+def forward_raw(
+    q,
+    k,
+    v,
+    q_blk,
+    k_blk,
+    q_valid,
+    k_valid,
+    scale: float,
+    k_new=None,
+    v_new=None,
+    *,
+    kvcache: bool = False,
+    workspace: torch.Tensor | None = None,
+    summary_ready: bool = False,
+    out: torch.Tensor | None = None,
+    want_lse: bool = True,
+):
+    """One forward through the C ABI.  Returns ``(out (B,Sq,H,D), lse (B,H,Sq) | None)``.
+
+    ``k``/``v`` are key segment 0; ``k_new``/``v_new`` (optional) segment 1.
+    ``workspace`` (uint8, device) may be passed to reuse the key-tile summary of
+    an earlier call with the same mask (``summary_ready=True``).
+    """
+    lib = _loader.require_library()
+    _check_inputs(q, k, v)
+    code, vec = _DTYPES[q.dtype]
+    b, sq, h, d = q.shape
+    sk0, hkv = k.shape[1], k.shape[2]
+    sk1 = 0 if k_new is None else k_new.shape[1]
+    q, k, v = _operand(q, vec), _operand(k, vec), _operand(v, vec)
+    if k_new is not None:
+        k_new, v_new = _operand(k_new, vec), _operand(v_new, vec)
+    q_blk, q_valid = _ids(q_blk, q_valid)
+    k_blk, k_valid = _ids(k_blk, k_valid)
+    if q_blk.shape != (b, sq) or k_blk.shape != (b, sk0 + sk1) or k_valid.shape != k_blk.shape:
+        raise RuntimeError(
+            f"block ids do not match q/k: q_blk {tuple(q_blk.shape)}, k_blk {tuple(k_blk.shape)}, "
+            f"expected {(b, sq)} and {(b, sk0 + sk1)}"
+        )
+    if out is None:
+        out = torch.empty((b, sq, h, d), dtype=q.dtype, device=q.device)
+    lse = torch.empty((b, h, sq), dtype=torch.float32, device=q.device) if want_lse else None
+    p = _loader.FwdParams()
+    p.q, p.k, p.v, p.k1, p.v1, p.o = _t4(q), _t4(k), _t4(v), _t4(k_new), _t4(v_new), _t4(out)
+    p.lse = lse.data_ptr() if lse is not None else None
+    p.q_blk, p.k_blk = q_blk.data_ptr(), k_blk.data_ptr()
+    p.q_valid, p.k_valid = q_valid.data_ptr(), k_valid.data_ptr()
+    p.B, p.Sq, p.Sk0, p.Sk1, p.H, p.Hkv, p.D = b, sq, sk0, sk1, h, hkv, d
+    p.dtype, p.scale = code, float(scale)
+    p.summary_ready = 1 if summary_ready else 0
+    size_fn = lib.bcattn_fwd_kvcache_workspace_bytes if kvcache else lib.bcattn_fwd_workspace_bytes
+    need = size_fn(ctypes.byref(p))
+    if workspace is None or workspace.numel() < need:
+        if summary_ready:
+            raise RuntimeError("summary_ready needs the workspace of the earlier call")
+        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    p.workspace, p.workspace_bytes = workspace.data_ptr(), workspace.numel()
+    with torch.cuda.device(q.device):
+        fn = lib.bcattn_fwd_kvcache if kvcache else lib.bcattn_fwd
+        _check(fn(ctypes.byref(p), _stream(q.device)), lib)
+    return out, lse
+
+
+def backward_raw(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale: float):
+    """One backward through the C ABI.  Returns ``(dq, dk, dv)``."""
+    lib = _loader.require_library()
+    _check_inputs(q, k, v)
+    code, vec = _DTYPES[q.dtype]
+    b, sq, h, d = q.shape
+    sk, hkv = k.shape[1], k.shape[2]
+    q, k, v, out, d_out = (_operand(t, vec) for t in (q, k, v, out, d_out))
+    q_blk, q_valid = _ids(q_blk, q_valid)
+    k_blk, k_valid = _ids(k_blk, k_valid)
+    lse = lse.contiguous()
+    dq = torch.empty((b, sq, h, d), dtype=q.dtype, device=q.device)
+    dk = torch.empty((b, sk, hkv, d), dtype=q.dtype, device=q.device)
+    dv = torch.empty((b, sk, hkv, d), dtype=q.dtype, device=q.device)
+    p = _loader.BwdParams()
+    p.q, p.k, p.v, p.o, p.d_o = _t4(q), _t4(k), _t4(v), _t4(out), _t4(d_out)
+    p.dq, p.dk, p.dv = _t4(dq), _t4(dk), _t4(dv)
+    p.lse = lse.data_ptr()
+    p.q_blk, p.k_blk = q_blk.data_ptr(), k_blk.data_ptr()
+    p.q_valid, p.k_valid = q_valid.data_ptr(), k_valid.data_ptr()
+    p.B, p.Sq, p.Sk, p.H, p.Hkv, p.D = b, sq, sk, h, hkv, d
+    p.dtype, p.scale = code, float(scale)
+    need = lib.bcattn_bwd_workspace_bytes(ctypes.byref(p))
+    workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    p.workspace, p.workspace_bytes = workspace.data_ptr(), workspace.numel()
+    with torch.cuda.device(q.device):
+        _check(lib.bcattn_bwd(ctypes.byref(p), _stream(q.device)), lib)
+    return dq, dk, dv
+
+
+# --------------------------------------------------------------------------- #
+# torch custom ops (autograd + fake implementations, so torch.compile can trace)
+# --------------------------------------------------------------------------- #
+@torch.library.custom_op("bcattn::fwd", mutates_args=())
+def _op_fwd(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    q_blk: torch.Tensor,
+    k_blk: torch.Tensor,
+    q_valid: torch.Tensor,
+    k_valid: torch.Tensor,
+    scale: float,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    out, lse = forward_raw(q, k, v, q_blk, k_blk, q_valid, k_valid, scale)
+    return out, lse
+
+
+@_op_fwd.register_fake
+def _(q, k, v, q_blk, k_blk, q_valid, k_valid, scale):
+    b, sq, h, d = q.shape
+    return q.new_empty((b, sq, h, d)), q.new_empty((b, h, sq), dtype=torch.float32)
+
+
+@torch.library.custom_op("bcattn::fwd_kvcache", mutates_args=())
+def _op_fwd_kvcache(
+    q: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    k_new: torch.Tensor,
+    v_new: torch.Tensor,
+    q_blk: torch.Tensor,
+    k_blk: torch.Tensor,
+    q_valid: torch.Tensor,
+    k_valid: torch.Tensor,
+    scale: float,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    out, lse = forward_raw(
+        q, k_cache, v_cache, q_blk, k_blk, q_valid, k_valid, scale, k_new, v_new, kvcache=True
+    )
+    return out, lse
+
+
+@_op_fwd_kvcache.register_fake
+def _(q, k_cache, v_cache, k_new, v_new, q_blk, k_blk, q_valid, k_valid, scale):
+    b, sq, h, d = q.shape
+    return q.new_empty((b, sq, h, d)), q.new_empty((b, h, sq), dtype=torch.float32)
+
+
+@torch.library.custom_op("bcattn::bwd", mutates_args=())
+def _op_bwd(
+    d_out: torch.Tensor,
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    out: torch.Tensor,
+    lse: torch.Tensor,
+    q_blk: torch.Tensor,
+    k_blk: torch.Tensor,
+    q_valid: torch.Tensor,
+    k_valid: torch.Tensor,
+    scale: float,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    return backward_raw(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale)
+
+
+@_op_bwd.register_fake
+def _(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale):
+    return (
+        q.new_empty(q.shape),
+        k.new_empty(k.shape),
+        v.new_empty(v.shape),
+    )
+
+
+def _fwd_setup(ctx, inputs, output):
+    q, k, v, q_blk, k_blk, q_valid, k_valid, scale = inputs
+    out, lse = output
+    ctx.save_for_backward(q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid)
+    ctx.scale = scale
+
+
+def _fwd_backward(ctx, d_out, _d_lse):
+    q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid = ctx.saved_tensors
+    dq, dk, dv = _op_bwd(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, ctx.scale)
+    return dq, dk, dv, None, None, None, None, None
+
+
+_op_fwd.register_autograd(_fwd_backward, setup_context=_fwd_setup)
+
+
+def _kvc_setup(ctx, inputs, output):
+    q, k_cache, v_cache, k_new, v_new, q_blk, k_blk, q_valid, k_valid, scale = inputs
+    out, lse = output
+    ctx.save_for_backward(q, k_cache, v_cache, k_new, v_new, out, lse, q_blk, k_blk, q_valid, k_valid)
+    ctx.scale = scale
+
+
+def _kvc_backward(ctx, d_out, _d_lse):
+    q, k_cache, v_cache, k_new, v_new, out, lse, q_blk, k_blk, q_valid, k_valid = ctx.saved_tensors
+    n0 = k_cache.shape[1]
+    k = torch.cat([k_cache, k_new], dim=1)
+    v = torch.cat([v_cache, v_new], dim=1)
+    dq, dk, dv = _op_bwd(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, ctx.scale)
+    return dq, dk[:, :n0], dv[:, :n0], dk[:, n0:], dv[:, n0:], None, None, None, None, None
+
+
+_op_fwd_kvcache.register_autograd(_kvc_backward, setup_context=_kvc_setup)
+
+
+def _needs_graph(*ts: torch.Tensor) -> bool:
+    return torch.compiler.is_compiling() or (torch.is_grad_enabled() and any(t.requires_grad for t in ts))
+
+
+def flash_attn_blockmask(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    q_blk: torch.Tensor,
+    k_blk: torch.Tensor,
+    q_valid: torch.Tensor,
+    k_valid: torch.Tensor,
+    scale: float,
+) -> torch.Tensor:
+    """Block-causal flash attention, ``(B,Sq,H,D), (B,Sk,Hkv,D) x2 -> (B,Sq,H,D)``.
+
+    Same signature and semantics as the reference's ``flash_attn_blockmask``
+    (``src/opentau/policies/flash_attn_cuda/__init__.py:146-171``).  Rows with no
+    visible key come back as zeros.  Raises ``RuntimeError`` when the kernels are
+    unavailable.
+    """
+    if _needs_graph(q, k, v):
+        return _op_fwd(q, k, v, q_blk, k_blk, q_valid, k_valid, float(scale))[0]
+    return forward_raw(q, k, v, q_blk, k_blk, q_valid, k_valid, scale, want_lse=False)[0]
+
+
+def flash_attn_blockmask_kvcache(
+    q: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    k_new: torch.Tensor,
+    v_new: torch.Tensor,
+    q_blk: torch.Tensor,
+    k_blk: torch.Tensor,
+    q_valid: torch.Tensor,
+    k_valid: torch.Tensor,
+    scale: float,
+) -> torch.Tensor:
+    """Attention of a few query rows over ``[k_cache ; k_new]`` without the concat.
+
+    Numerically the same as
+    ``flash_attn_blockmask(q, cat(k_cache, k_new), cat(v_cache, v_new), ...)`` with
+    ``k_blk``/``k_valid`` covering the concatenation (cached columns carry
+    ``INT_BLK_MIN``), which is what the reference computes per layer and denoise
+    step (``src/opentau/policies/pi05/paligemma_with_expert.py:742-768``).
+    """
+    if _needs_graph(q, k_cache, v_cache, k_new, v_new):
+        return _op_fwd_kvcache(q, k_cache, v_cache, k_new, v_new, q_blk, k_blk, q_valid, k_valid, float(scale))[0]
+    return forward_raw(
+        q, k_cache, v_cache, q_blk, k_blk, q_valid, k_valid, scale, k_new, v_new, kvcache=True, want_lse=False
+    )[0]

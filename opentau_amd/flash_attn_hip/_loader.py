@@ -1,0 +1,204 @@
+"""Loads ``libbcattn.so`` (HIP kernels behind a C ABI) with ctypes.
+
+Counterpart of ``src/opentau/policies/flash_attn_cuda/_loader.py:42-103``: lazy,
+once per process, lock-guarded, with ``is_available()`` / ``load_error()`` and an
+environment kill-switch.  Unlike the reference nothing is compiled at run time:
+the library is built ahead of time (``make -C opentau_amd/csrc``) and there is
+**no fallback** — when the library or a GPU is missing, calls raise.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from pathlib import Path
+
+CSRC = Path(__file__).resolve().parent.parent / "csrc"
+LIB_PATH = CSRC / "libbcattn.so"
+ABI_VERSION = 1
+
+# status codes of include/bcattn.h
+OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_LAUNCH = 0, -1, -2, -3, -4
+DTYPE_F32, DTYPE_BF16 = 0, 1
+
+EXPORTS = (
+    "bcattn_abi_version",
+    "bcattn_last_error",
+    "bcattn_fwd_workspace_bytes",
+    "bcattn_fwd_kvcache_workspace_bytes",
+    "bcattn_bwd_workspace_bytes",
+    "bcattn_fwd",
+    "bcattn_fwd_kvcache",
+    "bcattn_bwd",
+)
+
+
+class Tensor4(ctypes.Structure):
+    """``bcattn_tensor``."""
+
+    _fields_ = [
+        ("ptr", ctypes.c_void_p),
+        ("stride_b", ctypes.c_int64),
+        ("stride_s", ctypes.c_int64),
+        ("stride_h", ctypes.c_int64),
+    ]
+
+
+class FwdParams(ctypes.Structure):
+    """``bcattn_fwd_params``."""
+
+    _fields_ = [
+        ("q", Tensor4),
+        ("k", Tensor4),
+        ("v", Tensor4),
+        ("k1", Tensor4),
+        ("v1", Tensor4),
+        ("o", Tensor4),
+        ("lse", ctypes.c_void_p),
+        ("q_blk", ctypes.c_void_p),
+        ("k_blk", ctypes.c_void_p),
+        ("q_valid", ctypes.c_void_p),
+        ("k_valid", ctypes.c_void_p),
+        ("B", ctypes.c_int32),
+        ("Sq", ctypes.c_int32),
+        ("Sk0", ctypes.c_int32),
+        ("Sk1", ctypes.c_int32),
+        ("H", ctypes.c_int32),
+        ("Hkv", ctypes.c_int32),
+        ("D", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("scale", ctypes.c_float),
+        ("summary_ready", ctypes.c_int32),
+        ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_size_t),
+    ]
+
+
+class BwdParams(ctypes.Structure):
+    """``bcattn_bwd_params``."""
+
+    _fields_ = [
+        ("q", Tensor4),
+        ("k", Tensor4),
+        ("v", Tensor4),
+        ("o", Tensor4),
+        ("d_o", Tensor4),
+        ("dq", Tensor4),
+        ("dk", Tensor4),
+        ("dv", Tensor4),
+        ("lse", ctypes.c_void_p),
+        ("q_blk", ctypes.c_void_p),
+        ("k_blk", ctypes.c_void_p),
+        ("q_valid", ctypes.c_void_p),
+        ("k_valid", ctypes.c_void_p),
+        ("B", ctypes.c_int32),
+        ("Sq", ctypes.c_int32),
+        ("Sk", ctypes.c_int32),
+        ("H", ctypes.c_int32),
+        ("Hkv", ctypes.c_int32),
+        ("D", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("scale", ctypes.c_float),
+        ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_size_t),
+    ]
+
+
+_lock = threading.Lock()
+_lib = None
+_load_attempted = False
+_load_error: str | None = None
+
+
+def _bind(lib: ctypes.CDLL) -> ctypes.CDLL:
+    lib.bcattn_abi_version.restype = ctypes.c_int
+    lib.bcattn_abi_version.argtypes = []
+    lib.bcattn_last_error.restype = ctypes.c_char_p
+    lib.bcattn_last_error.argtypes = []
+    for name, st in (
+        ("bcattn_fwd_workspace_bytes", FwdParams),
+        ("bcattn_fwd_kvcache_workspace_bytes", FwdParams),
+        ("bcattn_bwd_workspace_bytes", BwdParams),
+    ):
+        fn = getattr(lib, name)
+        fn.restype = ctypes.c_size_t
+        fn.argtypes = [ctypes.POINTER(st)]
+    for name, st in (("bcattn_fwd", FwdParams), ("bcattn_fwd_kvcache", FwdParams), ("bcattn_bwd", BwdParams)):
+        fn = getattr(lib, name)
+        fn.restype = ctypes.c_int
+        fn.argtypes = [ctypes.POINTER(st), ctypes.c_void_p]
+    return lib
+
+
+def load_library() -> ctypes.CDLL:
+    """dlopen the built library and bind its entry points (no GPU needed).
+
+    Raises ``RuntimeError`` when the library is missing, misses a symbol, or
+    reports another ABI version.
+    """
+    if os.environ.get("OPENTAU_DISABLE_FLASH_HIP", "0") == "1":
+        raise RuntimeError("flash_hip disabled via OPENTAU_DISABLE_FLASH_HIP=1")
+    if not LIB_PATH.exists():
+        raise RuntimeError(f"{LIB_PATH} not built; run `make -C {CSRC}`")
+    lib = ctypes.CDLL(str(LIB_PATH))
+    missing = [s for s in EXPORTS if not hasattr(lib, s)]
+    if missing:
+        raise RuntimeError(f"{LIB_PATH} lacks symbols: {missing}")
+    _bind(lib)
+    got = lib.bcattn_abi_version()
+    if got != ABI_VERSION:
+        raise RuntimeError(f"{LIB_PATH} has ABI version {got}, binding expects {ABI_VERSION}")
+    return lib
+
+
+def get_library():
+    """The loaded library, or ``None`` when it is unavailable (see ``load_error``).
+
+    Memoised and thread-safe: loading is attempted at most once per process.
+    """
+    global _lib, _load_attempted, _load_error
+    if _lib is not None:
+        return _lib
+    if _load_attempted:
+        return None
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if _load_attempted:
+            return None
+        try:
+            import torch
+
+            if not torch.cuda.is_available():
+                raise RuntimeError("no HIP device is available")
+            _lib = load_library()
+        except Exception as exc:  # noqa: BLE001
+            _load_error = f"{type(exc).__name__}: {exc}"
+        finally:
+            _load_attempted = True
+    return _lib
+
+
+def require_library():
+    lib = get_library()
+    if lib is None:
+        raise RuntimeError(f"flash_hip kernel unavailable: {_load_error}")
+    return lib
+
+
+def is_available() -> bool:
+    """True when the library loaded and a HIP device is present."""
+    return get_library() is not None
+
+
+def load_error() -> str | None:
+    """Why loading failed, or ``None``."""
+    get_library()
+    return _load_error
+
+
+def _reset_for_tests() -> None:
+    global _lib, _load_attempted, _load_error
+    with _lock:
+        _lib, _load_attempted, _load_error = None, False, None

@@ -1,0 +1,175 @@
+"""Seeded synthetic workloads of the block-causal attention path.
+
+The five shapes are the attention calls of the policies this path serves:
+
+* ``c1``  one fp32 forward, B1 H8 Hkv1 D256, 304 prefix tokens + 50 action tokens
+* ``c2``  pi0.5 inference, bf16 B8 H8 Hkv1 D256: 968-token prefix (768 image +
+  200 text, 20..200 valid) then 50-token suffix steps over the cached prefix
+* ``c3``  pi0.5 training, bf16 B32 H8 Hkv1 D256: 640 prefix (512 image + 128
+  text, 16..128 valid) + 64 causal tokens + 50-token block
+* ``c4``  pi0.6, bf16 B16 H8 Hkv4 D256: 1024 prefix (768 + 256 text, 32..256
+  valid) + 50-token block
+* ``c5``  cosmos3, bf16 B4 H64 Hkv8 D128: 4352 prefix (4096 + 256 text, 64..256
+  valid) + 50-token block
+
+Tensors are drawn on the CPU from one ``torch.Generator`` seeded ``1234 + id`` in
+the order q, k, v, dO, text lengths, in fp32, then cast and moved, so a CPU
+checker and the GPU kernels see bit-identical inputs.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import torch
+
+from .flash_attn_hip import make_att_block_ids
+
+
+@dataclass
+class Workload:
+    name: str
+    dtype: torch.dtype
+    B: int
+    H: int
+    Hkv: int
+    D: int
+    n_fixed: int  # always-valid prefix tokens (image / video)
+    n_text: int  # right-padded text slots
+    text_lo: int
+    text_hi: int
+    n_causal: int  # tokens that each open a block
+    n_action: int  # one final block
+    q: torch.Tensor = field(default=None, repr=False)
+    k: torch.Tensor = field(default=None, repr=False)
+    v: torch.Tensor = field(default=None, repr=False)
+    d_out: torch.Tensor = field(default=None, repr=False)
+    pad: torch.Tensor = field(default=None, repr=False)
+    att: torch.Tensor = field(default=None, repr=False)
+    text_len: torch.Tensor = field(default=None, repr=False)
+
+    @property
+    def S(self) -> int:  # noqa: N802
+        return self.n_fixed + self.n_text + self.n_causal + self.n_action
+
+    @property
+    def n_prefix(self) -> int:
+        return self.n_fixed + self.n_text
+
+    @property
+    def scale(self) -> float:
+        return self.D**-0.5
+
+    def block_ids(self):
+        return make_att_block_ids(self.pad, self.att)
+
+    def pairs(self) -> int:
+        """Number of (query, key) pairs that attend, summed over the batch."""
+        q_blk, k_blk, q_valid, k_valid = (t.cpu() for t in self.block_ids())
+        total = 0
+        for b in range(self.B):
+            kb = k_blk[b][k_valid[b]].sort().values
+            qb = q_blk[b][q_valid[b]]
+            total += int(torch.searchsorted(kb, qb, right=True).sum())
+        return total
+
+    def to(self, device) -> "Workload":
+        for name in ("q", "k", "v", "d_out", "pad", "att", "text_len"):
+            t = getattr(self, name)
+            if t is not None:
+                setattr(self, name, t.to(device))
+        return self
+
+
+_SPECS = {
+    "c1": dict(dtype=torch.float32, B=1, H=8, Hkv=1, D=256, n_fixed=304, n_text=0, text_lo=0, text_hi=0,
+               n_causal=0, n_action=50),
+    "c2": dict(dtype=torch.bfloat16, B=8, H=8, Hkv=1, D=256, n_fixed=768, n_text=200, text_lo=20,
+               text_hi=200, n_causal=0, n_action=50),
+    "c3": dict(dtype=torch.bfloat16, B=32, H=8, Hkv=1, D=256, n_fixed=512, n_text=128, text_lo=16,
+               text_hi=128, n_causal=64, n_action=50),
+    "c4": dict(dtype=torch.bfloat16, B=16, H=8, Hkv=4, D=256, n_fixed=768, n_text=256, text_lo=32,
+               text_hi=256, n_causal=0, n_action=50),
+    "c5": dict(dtype=torch.bfloat16, B=4, H=64, Hkv=8, D=128, n_fixed=4096, n_text=256, text_lo=64,
+               text_hi=256, n_causal=0, n_action=50),
+}
+_IDS = {"c1": 1, "c2": 2, "c3": 3, "c4": 4, "c5": 5}
+
+
+def spec(name: str) -> dict:
+    return dict(_SPECS[name])
+
+
+def make_workload(name: str, *, batch: int | None = None, with_grad: bool = True) -> Workload:
+    """Build workload ``name`` ("c1".."c5") on the CPU; ``batch`` overrides B (same seed)."""
+    sp = spec(name)
+    if batch is not None:
+        sp["B"] = batch
+    w = Workload(name=name, **sp)
+    gen = torch.Generator(device="cpu").manual_seed(1234 + _IDS[name])
+    s = w.S
+    w.q = torch.randn(w.B, s, w.H, w.D, generator=gen).to(w.dtype)
+    w.k = torch.randn(w.B, s, w.Hkv, w.D, generator=gen).to(w.dtype)
+    w.v = torch.randn(w.B, s, w.Hkv, w.D, generator=gen).to(w.dtype)
+    if with_grad:
+        w.d_out = torch.randn(w.B, s, w.H, w.D, generator=gen).to(w.dtype)
+    if w.n_text:
+        w.text_len = torch.randint(w.text_lo, w.text_hi + 1, (w.B,), generator=gen)
+    else:
+        w.text_len = torch.zeros(w.B, dtype=torch.long)
+    pad = torch.ones(w.B, s, dtype=torch.bool)
+    if w.n_text:
+        pos = torch.arange(w.n_text)[None, :]
+        pad[:, w.n_fixed : w.n_fixed + w.n_text] = pos < w.text_len[:, None]
+    att = torch.zeros(w.B, s, dtype=torch.int32)
+    att[:, w.n_prefix : w.n_prefix + w.n_causal] = 1
+    att[:, w.n_prefix + w.n_causal] = 1
+    w.pad, w.att = pad, att
+    return w
+
+
+@dataclass
+class DenoiseWorkload:
+    """Prefix pass + suffix steps over the cached prefix K/V (``c2``; ``c4`` inference)."""
+
+    name: str
+    base: Workload
+    layers: int
+    steps: int
+    # per layer: prefix q/k/v; per (layer, step): suffix q/k/v
+    prefix: list = field(default_factory=list, repr=False)
+    suffix: list = field(default_factory=list, repr=False)
+    prefix_ids: tuple = None
+    suffix_ids: tuple = None
+
+
+def make_denoise_workload(name: str = "c2", *, layers: int = 18, steps: int = 10, device="cpu",
+                          distinct: int | None = None) -> DenoiseWorkload:
+    """Inputs of one ``sample_actions``: ``layers`` prefix calls, ``layers*steps`` suffix calls.
+
+    ``distinct`` bounds how many different suffix input sets are drawn (they are
+    cycled); ``None`` draws one per (layer, step).  Prefix mask: all of block 0;
+    suffix mask: cached columns (``INT_BLK_MIN``, validity = prefix padding) then
+    one 50-token block.
+    """
+    base = make_workload(name, with_grad=False)
+    gen = torch.Generator(device="cpu").manual_seed(4321 + _IDS[name])
+    b, h, hkv, d, npre, nact = base.B, base.H, base.Hkv, base.D, base.n_prefix, base.n_action
+    dw = DenoiseWorkload(name=name, base=base, layers=layers, steps=steps)
+    pre_pad = base.pad[:, :npre].contiguous()
+    pre_att = torch.zeros(b, npre, dtype=torch.int32)
+    dw.prefix_ids = tuple(t.to(device) for t in make_att_block_ids(pre_pad, pre_att))
+    suf_pad = torch.ones(b, nact, dtype=torch.bool)
+    suf_att = torch.zeros(b, nact, dtype=torch.int32)
+    suf_att[:, 0] = 1
+    dw.suffix_ids = tuple(t.to(device) for t in make_att_block_ids(suf_pad, suf_att, npre, pre_pad))
+
+    def draw(s, heads):
+        return torch.randn(b, s, heads, d, generator=gen).to(base.dtype).to(device)
+
+    for _ in range(layers):
+        dw.prefix.append((draw(npre, h), draw(npre, hkv), draw(npre, hkv)))
+    n_suf = layers * steps if distinct is None else min(distinct, layers * steps)
+    for _ in range(n_suf):
+        dw.suffix.append((draw(nact, h), draw(nact, hkv), draw(nact, hkv)))
+    return dw

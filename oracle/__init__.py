@@ -1,0 +1,3 @@
+"""CPU oracle for the block-causal attention path. Test infrastructure only:
+imported by tests/, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py``; never by the product package."""
