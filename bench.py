@@ -1,0 +1,258 @@
+#!/usr/bin/env python3
+"""Benchmark of the block-causal attention path on one MI355X.
+
+One step = one forward + backward of the cosmos3-shape attention call (bf16, B4
+H64 Hkv8 D128, S = 4352 prefix + 50 action tokens, seeded synthetic inputs)
+through the C ABI.  ``value`` is TFLOP/s on unmasked FLOPs only
+(``14 * D * H * pairs`` per step: 4 for the forward's two products, 10 for the
+backward's five), inputs resident in HBM.  Every part of the step is bracketed
+by HIP events on the launch stream inside the timed region, which gives the
+per-kernel durations behind ``roofline``.  The pi0.5 denoise attention (18
+prefix calls + 180 cached-suffix calls at B=8) is timed after it and reported
+under ``denoise``.  ``cpu_baseline`` is the eager CPU oracle on a bounded slice
+of the same workload.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-denoise]
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-denoise", action="store_true", help="skip the pi0.5 denoise leg")
+    ap.add_argument("--workload", default="c5", choices=["c3", "c4", "c5"])
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
+              file=sys.stderr)
+        return 2
+
+    import torch
+
+    from opentau_amd import flash_attn_hip as fa
+    from opentau_amd.flash_attn_hip import _loader
+    from opentau_amd.workloads import make_denoise_workload, make_workload
+
+    if not fa.is_available():
+        print(f"bench.py: HIP kernels unavailable: {fa.load_error()}", file=sys.stderr)
+        return 1
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    w = make_workload(args.workload)
+    pairs = w.pairs()
+    unit = w.D * w.H * pairs  # FLOPs per "GEMM unit" / 2
+    ids = [t.to(dev) for t in w.block_ids()]
+    q, k, v, go = (t.to(dev) for t in (w.q, w.k, w.v, w.d_out))
+    grads = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v))
+    out = torch.empty_like(q)
+    ws_f = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
+    ws_b = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
+    parts = ("fwd", "bwd_delta", "bwd_dq", "bwd_dkv")
+
+    def step(ev=None, ready=True):
+        if ev:
+            ev[0].record()
+        _, lse = fa.forward_raw(q, k, v, *ids, w.scale, workspace=ws_f, summary_ready=ready, out=out)
+        if ev:
+            ev[1].record()
+        for n, st in enumerate((_loader.BWD_DELTA, _loader.BWD_DQ, _loader.BWD_DKV)):
+            fa.backward_raw(go, q, k, v, out, lse, *ids, w.scale, stages=st, workspace=ws_b,
+                            summary_ready=ready, grads=grads)
+            if ev:
+                ev[2 + n].record()
+
+    step(ready=False)  # fills the tile summaries once; the masks do not change between steps
+    for _ in range(args.warmup):
+        step()
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s in range(args.steps):
+        step(events[s])
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    part_ms = {p: sum(e[i].elapsed_time(e[i + 1]) for e in events) / args.steps for i, p in enumerate(parts)}
+    tflops = 14 * unit / (ms_per_step * 1e-3) / 1e12
+
+    # Unmasked FLOPs each kernel is credited with.  The backward's five products
+    # (10*unit) are S, dP, dV, dK, dQ; S and dP are formed in both backward kernels
+    # and are credited half to each, so the parts sum to the 14*unit of the step.
+    credit = {"fwd": 4 * unit, "bwd_delta": 0, "bwd_dq": 4 * unit, "bwd_dkv": 6 * unit}
+    dom = max(("fwd", "bwd_dq", "bwd_dkv"), key=lambda p: part_ms[p])
+    achieved = credit[dom] / (part_ms[dom] * 1e-3) / 1e12
+    roofline = {
+        "bound": "mfma",
+        "kernel": {"fwd": "fwd_bf16_kernel", "bwd_dq": "bwd_dq_kernel", "bwd_dkv": "bwd_dkv_kernel"}[dom],
+        "achieved": round(achieved, 2),
+        "peak": PEAK_BF16_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+        "traffic": None,
+        "kernel_ms": {p: round(part_ms[p], 4) for p in parts},
+        "kernel_tflops": {p: round(credit[p] / (part_ms[p] * 1e-3) / 1e12, 2) for p in parts if credit[p]},
+        "step_frac": round(tflops / PEAK_BF16_TFLOPS, 4),
+    }
+
+    result = {
+        "metric": "block-causal attn fwd+bwd TFLOP/s on unmasked FLOPs (cosmos3 shape, 1 GPU)",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{w.name}: bf16 fwd+bwd B{w.B} H{w.H} Hkv{w.Hkv} D{w.D} S{w.S} "
+                        f"({w.n_prefix} prefix in block 0, text valid {w.text_lo}..{w.text_hi}, "
+                        f"{w.n_causal} causal, {w.n_action}-token action block)",
+            "unmasked_pairs": pairs,
+            "flops_per_step": 14 * unit,
+            "pct_of_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2),
+        },
+        "roofline": roofline,
+    }
+
+    if not args.no_denoise:
+        result["denoise"] = bench_denoise(torch, fa, make_denoise_workload, dev)
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(torch, make_workload, args.workload)
+    print(json.dumps(result))
+    return 0
+
+
+def bench_denoise(torch, fa, make_denoise_workload, dev):
+    """pi0.5 inference attention: 18 prefix calls, then 10 steps x 18 cached-suffix calls."""
+    layers, steps = 18, 10
+    dw = make_denoise_workload("c2", layers=layers, steps=steps, device=dev, distinct=36)
+    w = dw.base
+    npre, nact = w.n_prefix, w.n_action
+    scale = w.scale
+    pre_ids, suf_ids = dw.prefix_ids, dw.suffix_ids
+    caches = [(kk[:, :npre], vv[:, :npre]) for (_, kk, vv) in dw.prefix]
+    ws_p = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
+    ws_s = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
+    out_p = torch.empty_like(dw.prefix[0][0])
+    out_s = torch.empty_like(dw.suffix[0][0])
+
+    def run(ev=None):
+        if ev:
+            ev[0].record()
+        for li in range(layers):
+            qq, kk, vv = dw.prefix[li]
+            fa.forward_raw(qq, kk, vv, *pre_ids, scale, workspace=ws_p, summary_ready=li > 0, out=out_p,
+                           want_lse=False)
+        if ev:
+            ev[1].record()
+        n = 0
+        for _ in range(steps):
+            for li in range(layers):
+                qs, kn, vn = dw.suffix[n % len(dw.suffix)]
+                kc, vc = caches[li]
+                fa.forward_raw(qs, kc, vc, *suf_ids, scale, kn, vn, kvcache=True, workspace=ws_s,
+                               summary_ready=n > 0, out=out_s, want_lse=False)
+                n += 1
+        if ev:
+            ev[2].record()
+
+    for _ in range(2):
+        run()
+    reps = 5
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(reps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for r in range(reps):
+        run(evs[r])
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / reps
+    pre_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / reps
+    suf_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / reps
+    valid = w.pad[:, :npre].sum().item()  # valid cached keys over the batch
+    kv_bytes = 2 * (valid + w.B * nact) * w.Hkv * w.D * 2
+    qo_bytes = 2 * w.B * nact * w.H * w.D * 2
+    id_bytes = w.B * (npre + 2 * nact) * 5
+    bytes_call = kv_bytes + qo_bytes + id_bytes
+    suf_call_us = suf_ms * 1e3 / (layers * steps)
+    gbps = bytes_call / (suf_call_us * 1e-6) / 1e9
+    pairs_pre = int((w.pad[:, :npre].sum(1) ** 2).sum())
+    pre_tflops = 4 * w.D * w.H * pairs_pre * layers / (pre_ms * 1e-3) / 1e12
+    return {
+        "workload": f"c2: pi0.5 inference bf16 B{w.B} H{w.H} Hkv{w.Hkv} D{w.D}, {layers} prefix calls "
+                    f"(S{npre}) + {steps}x{layers} suffix calls (Sq{nact}, Sk{npre + nact})",
+        "total_ms": round(pre_ms + suf_ms, 3),
+        "wall_ms": round(wall_ms, 3),
+        "prefix_ms": round(pre_ms, 3),
+        "prefix_tflops": round(pre_tflops, 1),
+        "suffix_ms": round(suf_ms, 3),
+        "suffix_us_per_call": round(suf_call_us, 2),
+        "suffix_algorithmic_bytes_per_call": int(bytes_call),
+        "suffix_GBps": round(gbps, 1),
+        "suffix_hbm_frac": round(gbps / PEAK_HBM_GBPS, 4),
+    }
+
+
+def cpu_baseline(torch, make_workload, name, budget_s=12.0):
+    """The eager CPU oracle (reference algorithm) on a bounded part of the same workload.
+
+    The workload is walked one (sample, kv head) slice at a time -- the kv head's
+    K/V with the query heads of its group, forward + backward by autograd -- until
+    about ``budget_s`` seconds of CPU work are done; the rate is unmasked FLOPs of
+    the slices done over the time they took.
+    """
+    from oracle import eager
+
+    w = make_workload(name)
+    grp = w.H // w.Hkv
+    ids = w.block_ids()
+    cores = torch.get_num_threads()
+    flops, dt, done = 0, 0.0, 0
+    for b in range(w.B):
+        sl = [t[b : b + 1] for t in ids]
+        pairs_b = int(eager.dense_mask_from_block_ids(*sl).sum())
+        for hk in range(w.Hkv):
+            hs = slice(hk * grp, (hk + 1) * grp)
+            q, go = w.q[b : b + 1, :, hs], w.d_out[b : b + 1, :, hs]
+            k, v = w.k[b : b + 1, :, hk : hk + 1], w.v[b : b + 1, :, hk : hk + 1]
+            t0 = time.perf_counter()
+            eager.eager_grads(q, k, v, go, *sl, w.scale)
+            dt += time.perf_counter() - t0
+            flops += 14 * w.D * grp * pairs_b
+            done += 1
+            if dt >= budget_s:
+                break
+        if dt >= budget_s:
+            break
+    return {
+        "value": round(flops / dt / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "seconds": round(dt, 2),
+        "sample": f"{name}: first {done} of {w.B * w.Hkv} (sample, kv head) slices, each the kv head with its "
+                  f"{grp} query heads, eager fwd+bwd by autograd, {flops / 1e9:.0f} GFLOP unmasked; "
+                  f"torch CPU {cores} threads of {os.cpu_count()} cpus",
+    }
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -104,9 +104,23 @@ typedef struct bcattn_bwd_params {
   int32_t B, Sq, Sk, H, Hkv, D;
   int32_t dtype;
   float scale;
+  /*
+   * Which parts to run, a bit set: BCATTN_BWD_DELTA (the row sums of O*dO, kept in
+   * the workspace), BCATTN_BWD_DQ, BCATTN_BWD_DKV; 0 means all three.  dQ and
+   * dK/dV read the delta (and the tile summaries) an earlier call left in the
+   * same workspace, so a caller that drops the key/value gradients (knowledge
+   * insulation detaches the cached K/V:
+   * src/opentau/policies/pi05/modeling_pi05.py:1752-1757) asks for
+   * DELTA|DQ only, and a profiler can time each part on its own.
+   */
+  int32_t stages;
+  /* Nonzero: the workspace already holds the tile summaries of these masks. */
+  int32_t summary_ready;
   void *workspace;
   size_t workspace_bytes;
 } bcattn_bwd_params;
+
+enum bcattn_bwd_stage { BCATTN_BWD_DELTA = 1, BCATTN_BWD_DQ = 2, BCATTN_BWD_DKV = 4 };
 
 /* Replaces nothing in the reference; version handshake for the binding. */
 int bcattn_abi_version(void);

@@ -190,7 +190,12 @@ int bcattn_fwd_kvcache(const bcattn_fwd_params *p, void *stream) {
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   FwdArgs a = fwd_args(p);
   char *ws = reinterpret_cast<char *>(p->workspace);
-  a.ksum = reinterpret_cast<tile_summary_t *>(ws);
+  tile_summary_t *ks = reinterpret_cast<tile_summary_t *>(ws);
+  if (!p->summary_ready) {
+    rc = launch_summary(p->k_blk, p->k_valid, a.B, a.Sk, ks, st);
+    if (rc) return fail(rc, "summary launch failed: %s", hipGetErrorString(hipGetLastError()));
+  }
+  a.ksum = ks;
   ws += summary_bytes(a.B, a.Sk);
   SplitArgs s;
   const size_t part = kvcache_workspace_bytes(a.B, a.Sq, a.Sk, a.H, a.Hkv, p->D, &s.nsplit);
@@ -239,6 +244,8 @@ int bcattn_bwd(const bcattn_bwd_params *p, void *stream) {
   a.q_blk = p->q_blk, a.k_blk = p->k_blk, a.q_valid = p->q_valid, a.k_valid = p->k_valid;
   a.B = p->B, a.Sq = p->Sq, a.Sk = p->Sk, a.H = p->H, a.Hkv = p->Hkv, a.G = p->H / p->Hkv;
   a.scale = p->scale;
+  a.stages = p->stages & (BCATTN_BWD_DELTA | BCATTN_BWD_DQ | BCATTN_BWD_DKV);
+  if (a.stages == 0) a.stages = BCATTN_BWD_DELTA | BCATTN_BWD_DQ | BCATTN_BWD_DKV;
   char *ws = reinterpret_cast<char *>(p->workspace);
   tile_summary_t *ks = reinterpret_cast<tile_summary_t *>(ws);
   ws += summary_bytes(a.B, a.Sk);
@@ -247,8 +254,9 @@ int bcattn_bwd(const bcattn_bwd_params *p, void *stream) {
   a.delta = reinterpret_cast<float *>(ws);
   a.ksum = ks;
   a.qsum = qs;
-  if ((rc = launch_summary(p->k_blk, p->k_valid, a.B, a.Sk, ks, st)) ||
-      (rc = launch_summary(p->q_blk, p->q_valid, a.B, a.Sq, qs, st)))
+  if (!p->summary_ready &&
+      ((rc = launch_summary(p->k_blk, p->k_valid, a.B, a.Sk, ks, st)) ||
+       (rc = launch_summary(p->q_blk, p->q_valid, a.B, a.Sq, qs, st))))
     return fail(rc, "summary launch failed");
   rc = p->dtype == BCATTN_BF16 ? launch_bwd_bf16(a, p->D, st) : launch_bwd_f32(a, p->D, st);
   if (rc) return fail(rc, "backward launch failed (D=%d dtype=%d)", p->D, p->dtype);

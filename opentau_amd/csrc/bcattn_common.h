@@ -170,6 +170,7 @@ struct BwdArgs {
   const tile_summary_t *qsum;  // (B, ceil(Sq/64))
   int B, Sq, Sk, H, Hkv, G;
   float scale;
+  int stages;  // bit set of bcattn_bwd_stage, never 0 here
 };
 
 // kernel launchers, one translation unit each
@@ -184,6 +185,7 @@ struct SplitArgs {
   float *part_o;   // (B, Hkv, nsplit, R, D) fp32, R = G*Sq
   float *part_ml;  // (B, Hkv, nsplit, R, 2) fp32: running max (raw scores), sum
   int nsplit;
+  int tiles_per_split;  // 64-key tiles per split
 };
 int launch_fwd_kvcache_bf16(const FwdArgs &a, const SplitArgs &s, int D, hipStream_t st);
 size_t kvcache_workspace_bytes(int B, int Sq, int Sk, int H, int Hkv, int D, int *nsplit_out);

@@ -14,8 +14,13 @@
 
 namespace bcattn {
 
-template <int D>
-__global__ __launch_bounds__(256) void fwd_bf16_kernel(const FwdArgs a) {
+//
+// SPLIT: the key tiles are divided over `nsplit` workgroups per row tile; each
+// writes its unnormalised fp32 partial (O, running max, sum) and
+// `fwd_combine_kernel` merges them.  This is what lets a handful of
+// (batch, kv head) problems with few query rows fill the chip.
+template <int D, bool SPLIT>
+__global__ __launch_bounds__(256) void fwd_bf16_kernel(const FwdArgs a, const SplitArgs sp) {
   constexpr int BN = 64;
   constexpr int KP = RowTile<D>::kPitch;
   constexpr int DK = D / 16;   // contraction steps of K Q^T
@@ -39,6 +44,8 @@ __global__ __launch_bounds__(256) void fwd_bf16_kernel(const FwdArgs a) {
   int bid = blockIdx.x;
   const int tile = bid % ntile_r;
   bid /= ntile_r;
+  const int split = SPLIT ? bid % sp.nsplit : 0;
+  if (SPLIT) bid /= sp.nsplit;
   const int hk = bid % a.Hkv;
   const int b = bid / a.Hkv;
 
@@ -72,7 +79,9 @@ __global__ __launch_bounds__(256) void fwd_bf16_kernel(const FwdArgs a) {
   const int any_g = red_s[4] | red_s[5] | red_s[6] | red_s[7];
 
   const int Sk = a.Sk;
-  const int nt = any_g ? (Sk + BN - 1) / BN : 0;
+  const int nt_all = (Sk + BN - 1) / BN;
+  const int t_first = SPLIT ? split * sp.tiles_per_split : 0;
+  const int nt = !any_g ? 0 : (SPLIT ? min(nt_all, t_first + sp.tiles_per_split) : nt_all);
   const tile_summary_t *ksum = a.ksum + (int64_t)b * ((Sk + BN - 1) / BN);
 
   const bf16_t *k0b = reinterpret_cast<const bf16_t *>(a.k0.ptr) + b * a.k0.sb + hk * a.k0.sh;
@@ -153,7 +162,7 @@ __global__ __launch_bounds__(256) void fwd_bf16_kernel(const FwdArgs a) {
   float l = 0.f;        // this lane half's share of the running sum
   const float c = a.scale * kLog2e;
 
-  int t = next_needed(0);
+  int t = next_needed(t_first);
   if (t < nt) prefetch(t);
   while (t < nt) {
     stage();
@@ -232,6 +241,28 @@ __global__ __launch_bounds__(256) void fwd_bf16_kernel(const FwdArgs a) {
 
   // ---- epilogue ----------------------------------------------------------------
   l += swap32(l);
+  if (SPLIT) {
+    if (rowok) {
+      const int64_t prow = (((int64_t)b * a.Hkv + hk) * sp.nsplit + split) * R + r;
+      if (hh == 0) {
+        f32x2 ml;
+        ml[0] = qv ? m : -INFINITY;
+        ml[1] = qv ? l : 0.f;
+        *reinterpret_cast<f32x2 *>(sp.part_ml + 2 * prow) = ml;
+      }
+      float *po = sp.part_o + prow * D;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+          f32x4 w;
+#pragma unroll
+          for (int x = 0; x < 4; ++x) w[x] = o[db][4 * r4 + x];
+          *reinterpret_cast<f32x4 *>(po + 32 * db + 8 * r4 + 4 * hh) = w;
+        }
+    }
+    return;
+  }
   const bool has = qv && l > 0.f;
   const float inv = has ? 1.f / l : 0.f;
   if (rowok) {
@@ -250,24 +281,122 @@ __global__ __launch_bounds__(256) void fwd_bf16_kernel(const FwdArgs a) {
   }
 }
 
+// Merge the per-split partials: one thread per (packed row, 4 head_dim columns).
+template <int D>
+__global__ __launch_bounds__(256) void fwd_combine_kernel(const FwdArgs a, const SplitArgs sp) {
+  constexpr int TPR = D / 4;
+  const int R = a.G * a.Sq;
+  const int64_t total = (int64_t)a.B * a.Hkv * R;
+  const int64_t idx = (int64_t)blockIdx.x * (256 / TPR) + threadIdx.x / TPR;
+  const int c4 = threadIdx.x % TPR;
+  if (idx >= total) return;
+  const int r = (int)(idx % R);
+  const int64_t bh = idx / R;
+  const int hk = (int)(bh % a.Hkv);
+  const int b = (int)(bh / a.Hkv);
+  const int g = r / a.Sq, i = r - g * a.Sq, h = hk * a.G + g;
+  const float c = a.scale * kLog2e;
+  const int64_t p0 = bh * sp.nsplit * R + r;
+  float mx = -INFINITY;
+  for (int s = 0; s < sp.nsplit; ++s) mx = fmaxf(mx, sp.part_ml[2 * (p0 + (int64_t)s * R)]);
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  float lsum = 0.f;
+  if (mx != -INFINITY) {
+    for (int s = 0; s < sp.nsplit; ++s) {
+      const int64_t pr = p0 + (int64_t)s * R;
+      const f32x2 ml = *reinterpret_cast<const f32x2 *>(sp.part_ml + 2 * pr);
+      if (ml[0] == -INFINITY) continue;
+      const float w = fast_exp2((ml[0] - mx) * c);
+      lsum += w * ml[1];
+      const f32x4 po = *reinterpret_cast<const f32x4 *>(sp.part_o + pr * D + 4 * c4);
+#pragma unroll
+      for (int x = 0; x < 4; ++x) acc[x] += w * po[x];
+    }
+  }
+  const bool has = lsum > 0.f;
+  const float inv = has ? 1.f / lsum : 0.f;
+  bf16x4 w;
+#pragma unroll
+  for (int x = 0; x < 4; ++x) w[x] = (bf16_t)(acc[x] * inv);
+  bf16_t *optr = reinterpret_cast<bf16_t *>(a.o) + b * a.o_sb + (int64_t)i * a.o_ss + h * a.o_sh;
+  *reinterpret_cast<bf16x4 *>(optr + 4 * c4) = w;
+  if (a.lse != nullptr && c4 == 0)
+    a.lse[((int64_t)b * a.H + h) * a.Sq + i] = has ? mx * a.scale + __logf(lsum) : 0.f;
+}
+
 int launch_fwd_bf16(const FwdArgs &a, int D, hipStream_t st) {
   const int R = a.G * a.Sq;
   const int ntile_r = (R + 127) / 128;
   const dim3 grid((unsigned)(ntile_r * a.Hkv * a.B)), block(256);
+  const SplitArgs sp{nullptr, nullptr, 1, 0};
   switch (D) {
     case 64:
-      hipLaunchKernelGGL(fwd_bf16_kernel<64>, grid, block, 0, st, a);
+      hipLaunchKernelGGL((fwd_bf16_kernel<64, false>), grid, block, 0, st, a, sp);
       break;
     case 128:
-      hipLaunchKernelGGL(fwd_bf16_kernel<128>, grid, block, 0, st, a);
+      hipLaunchKernelGGL((fwd_bf16_kernel<128, false>), grid, block, 0, st, a, sp);
       break;
     case 256:
-      hipLaunchKernelGGL(fwd_bf16_kernel<256>, grid, block, 0, st, a);
+      hipLaunchKernelGGL((fwd_bf16_kernel<256, false>), grid, block, 0, st, a, sp);
       break;
     default:
       return BCATTN_ERR_UNSUPPORTED;
   }
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
+}
+
+// How many ways to split the key axis so that about 1.5 workgroups per CU exist.
+static void plan_split(int B, int Sq, int Sk, int H, int Hkv, int *nsplit, int *tps) {
+  const int R = (H / Hkv) * Sq;
+  const int base = B * Hkv * ((R + 127) / 128);
+  const int ntiles = (Sk + 63) / 64;
+  int want = (384 + base - 1) / base;
+  if (want < 1) want = 1;
+  if (want > ntiles) want = ntiles;
+  *tps = (ntiles + want - 1) / want;
+  *nsplit = (ntiles + *tps - 1) / *tps;
+}
+
+size_t kvcache_workspace_bytes(int B, int Sq, int Sk, int H, int Hkv, int D, int *nsplit_out) {
+  int ns, tps;
+  plan_split(B, Sq, Sk, H, Hkv, &ns, &tps);
+  *nsplit_out = ns;
+  if (ns <= 1) return 0;
+  const size_t R = (size_t)(H / Hkv) * Sq;
+  const size_t rows = (size_t)B * Hkv * ns * R;
+  return ((rows * (D + 2) * sizeof(float)) + 255) & ~(size_t)255;
+}
+
+template <int D>
+static int launch_split(const FwdArgs &a, const SplitArgs &sp, hipStream_t st) {
+  const int R = a.G * a.Sq;
+  const int ntile_r = (R + 127) / 128;
+  hipLaunchKernelGGL((fwd_bf16_kernel<D, true>), dim3((unsigned)(ntile_r * sp.nsplit * a.Hkv * a.B)),
+                     dim3(256), 0, st, a, sp);
+  constexpr int RPB = 256 / (D / 4);
+  const int64_t rows = (int64_t)a.B * a.Hkv * R;
+  hipLaunchKernelGGL(fwd_combine_kernel<D>, dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, a,
+                     sp);
+  return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
+}
+
+int launch_fwd_kvcache_bf16(const FwdArgs &a, const SplitArgs &sp_in, int D, hipStream_t st) {
+  SplitArgs sp = sp_in;
+  int ns, tps;
+  plan_split(a.B, a.Sq, a.Sk, a.H, a.Hkv, &ns, &tps);
+  if (ns <= 1) return launch_fwd_bf16(a, D, st);
+  sp.nsplit = ns;
+  sp.tiles_per_split = tps;
+  switch (D) {
+    case 64:
+      return launch_split<64>(a, sp, st);
+    case 128:
+      return launch_split<128>(a, sp, st);
+    case 256:
+      return launch_split<256>(a, sp, st);
+    default:
+      return BCATTN_ERR_UNSUPPORTED;
+  }
 }
 
 }  // namespace bcattn

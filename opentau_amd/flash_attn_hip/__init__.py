@@ -193,8 +193,13 @@ def forward_raw(
     return out, lse
 
 
-def backward_raw(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale: float):
-    """One backward through the C ABI.  Returns ``(dq, dk, dv)``."""
+def backward_raw(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale: float, *, stages: int = 0,
+                 workspace: torch.Tensor | None = None, summary_ready: bool = False, grads=None):
+    """One backward through the C ABI.  Returns ``(dq, dk, dv)``.
+
+    ``stages`` selects parts (``_loader.BWD_DELTA | BWD_DQ | BWD_DKV``; 0 = all); parts
+    run separately must share ``workspace`` (and ``grads``, the output triple).
+    """
     lib = _loader.require_library()
     _check_inputs(q, k, v)
     code, vec = _DTYPES[q.dtype]
@@ -204,9 +209,12 @@ def backward_raw(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale
     q_blk, q_valid = _ids(q_blk, q_valid)
     k_blk, k_valid = _ids(k_blk, k_valid)
     lse = lse.contiguous()
-    dq = torch.empty((b, sq, h, d), dtype=q.dtype, device=q.device)
-    dk = torch.empty((b, sk, hkv, d), dtype=q.dtype, device=q.device)
-    dv = torch.empty((b, sk, hkv, d), dtype=q.dtype, device=q.device)
+    if grads is not None:
+        dq, dk, dv = grads
+    else:
+        dq = torch.empty((b, sq, h, d), dtype=q.dtype, device=q.device)
+        dk = torch.empty((b, sk, hkv, d), dtype=q.dtype, device=q.device)
+        dv = torch.empty((b, sk, hkv, d), dtype=q.dtype, device=q.device)
     p = _loader.BwdParams()
     p.q, p.k, p.v, p.o, p.d_o = _t4(q), _t4(k), _t4(v), _t4(out), _t4(d_out)
     p.dq, p.dk, p.dv = _t4(dq), _t4(dk), _t4(dv)
@@ -215,8 +223,12 @@ def backward_raw(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale
     p.q_valid, p.k_valid = q_valid.data_ptr(), k_valid.data_ptr()
     p.B, p.Sq, p.Sk, p.H, p.Hkv, p.D = b, sq, sk, h, hkv, d
     p.dtype, p.scale = code, float(scale)
+    p.stages, p.summary_ready = int(stages), 1 if summary_ready else 0
     need = lib.bcattn_bwd_workspace_bytes(ctypes.byref(p))
-    workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    if workspace is None or workspace.numel() < need:
+        if summary_ready or (stages and not stages & _loader.BWD_DELTA):
+            raise RuntimeError("this call needs the workspace an earlier call filled")
+        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
     p.workspace, p.workspace_bytes = workspace.data_ptr(), workspace.numel()
     with torch.cuda.device(q.device):
         _check(lib.bcattn_bwd(ctypes.byref(p), _stream(q.device)), lib)

@@ -21,6 +21,7 @@ ABI_VERSION = 1
 # status codes of include/bcattn.h
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_LAUNCH = 0, -1, -2, -3, -4
 DTYPE_F32, DTYPE_BF16 = 0, 1
+BWD_DELTA, BWD_DQ, BWD_DKV = 1, 2, 4
 
 EXPORTS = (
     "bcattn_abi_version",
@@ -100,6 +101,8 @@ class BwdParams(ctypes.Structure):
         ("D", ctypes.c_int32),
         ("dtype", ctypes.c_int32),
         ("scale", ctypes.c_float),
+        ("stages", ctypes.c_int32),
+        ("summary_ready", ctypes.c_int32),
         ("workspace", ctypes.c_void_p),
         ("workspace_bytes", ctypes.c_size_t),
     ]
