@@ -34,15 +34,13 @@ __device__ __forceinline__ void load_units(bf16x8 (&reg)[TileUnits<D>::NU][4], c
   using T = TileUnits<D>;
 #pragma unroll
   for (int it = 0; it < T::NU; ++it) {
-    const int u = tid + 256 * it;
+    const int u = min(tid + 256 * it, T::UNITS - 1);
     const int dch = u % T::CPR, kg = u / T::CPR;
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
-      const int row = row0 + 4 * kg + x;
-      bf16x8 val = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (u < T::UNITS && row < nrows)
-        val = *reinterpret_cast<const bf16x8 *>(base + (int64_t)row * row_stride + dch * 8);
-      reg[it][x] = val;
+      const int row = row0 + 4 * kg + x, rc = min(row, nrows - 1);
+      const bf16x8 val = *reinterpret_cast<const bf16x8 *>(base + (int64_t)rc * row_stride + dch * 8);
+      reg[it][x] = keep_if(row < nrows, val);
     }
   }
 }
@@ -180,15 +178,15 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(const BwdArgs a) {
     for (int it = 0; it < VCH; ++it) {
       const int c = tid + 256 * it;
       const int row = c / CPR, col = c % CPR;
-      bf16x8 val = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (j0 + row < Sk)
-        val = *reinterpret_cast<const bf16x8 *>(vb_ + (int64_t)(j0 + row) * a.v.ss + col * 8);
-      vreg[it] = val;
+      const int jc = min(j0 + row, Sk - 1);
+      const bf16x8 val = *reinterpret_cast<const bf16x8 *>(vb_ + (int64_t)jc * a.v.ss + col * 8);
+      vreg[it] = keep_if(j0 + row < Sk, val);
     }
-    if (tid < BN) {
-      const int j = j0 + tid;
-      kbreg = kIntMax;
-      if (j < Sk && a.k_valid[(int64_t)b * Sk + j]) kbreg = a.k_blk[(int64_t)b * Sk + j];
+    {
+      const int j = j0 + (tid & (BN - 1)), jc = min(j, Sk - 1);
+      const int id = a.k_blk[(int64_t)b * Sk + jc];
+      const int ok = a.k_valid[(int64_t)b * Sk + jc];
+      kbreg = (j < Sk && ok != 0) ? id : kIntMax;
     }
   };
   auto stage = [&]() {
@@ -228,12 +226,21 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(const BwdArgs a) {
         for (int x = 0; x < 16; ++x) s[x] = 0.f, dp[x] = 0.f;
         const bf16_t *kp = Ks + (32 * mb + n) * KP + 8 * hh;
         const bf16_t *vp = Vs + (32 * mb + n) * KP + 8 * hh;
+        constexpr int KB = DK < 8 ? DK : 8;  // operand reads issued ahead of the products
 #pragma unroll
-        for (int ks = 0; ks < DK; ++ks)
-          s = mfma32(*reinterpret_cast<const bf16x8 *>(kp + 16 * ks), qf[ks], s);
+        for (int k0 = 0; k0 < DK; k0 += KB) {
+          bf16x8 fa[KB], fb[KB];
 #pragma unroll
-        for (int ks = 0; ks < DK; ++ks)
-          dp = mfma32(*reinterpret_cast<const bf16x8 *>(vp + 16 * ks), gof[ks], dp);
+          for (int ks = 0; ks < KB; ++ks) {
+            fa[ks] = *reinterpret_cast<const bf16x8 *>(kp + 16 * (k0 + ks));
+            fb[ks] = *reinterpret_cast<const bf16x8 *>(vp + 16 * (k0 + ks));
+          }
+#pragma unroll
+          for (int ks = 0; ks < KB; ++ks) {
+            s = mfma32(fa[ks], qf[k0 + ks], s);
+            dp = mfma32(fb[ks], gof[k0 + ks], dp);
+          }
+        }
         float ds[16];
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
@@ -362,15 +369,15 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
     const bf16_t *gb_ = reinterpret_cast<const bf16_t *>(a.d_o.ptr) + b * a.d_o.sb + h * a.d_o.sh;
     load_units<D>(qreg, qb_, a.q.ss, i0, Sq, tid);
     load_units<D>(greg, gb_, a.d_o.ss, i0, Sq, tid);
-    if (tid < BQ) {
-      const int i = i0 + tid;
-      lsereg = INFINITY, delreg = 0.f, qbreg = kIntMin;
-      if (i < Sq && a.q_valid[(int64_t)b * Sq + i]) {
-        const int64_t stat = ((int64_t)b * a.H + h) * Sq + i;
-        lsereg = a.lse[stat] * kLog2e;
-        delreg = a.delta[stat];
-        qbreg = a.q_blk[(int64_t)b * Sq + i];
-      }
+    {
+      const int i = i0 + (tid & (BQ - 1)), ic = min(i, Sq - 1);
+      const int64_t stat = ((int64_t)b * a.H + h) * Sq + ic;
+      const float lv = a.lse[stat], dl = a.delta[stat];
+      const int id = a.q_blk[(int64_t)b * Sq + ic];
+      const bool ok = i < Sq && a.q_valid[(int64_t)b * Sq + ic] != 0;
+      lsereg = ok ? lv * kLog2e : INFINITY;
+      delreg = ok ? dl : 0.f;
+      qbreg = ok ? id : kIntMin;
     }
   };
   auto stage = [&]() {
@@ -409,12 +416,21 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
         for (int x = 0; x < 16; ++x) s[x] = 0.f, dp[x] = 0.f;
         const bf16_t *qp = Qs + (32 * mb + n) * KP + 8 * hh;
         const bf16_t *gp = Gs + (32 * mb + n) * KP + 8 * hh;
+        constexpr int KB = DK < 8 ? DK : 8;
 #pragma unroll
-        for (int ks = 0; ks < DK; ++ks)
-          s = mfma32(*reinterpret_cast<const bf16x8 *>(qp + 16 * ks), kf[ks], s);
+        for (int k0 = 0; k0 < DK; k0 += KB) {
+          bf16x8 fa[KB], fb[KB];
 #pragma unroll
-        for (int ks = 0; ks < DK; ++ks)
-          dp = mfma32(*reinterpret_cast<const bf16x8 *>(gp + 16 * ks), vf[ks], dp);
+          for (int ks = 0; ks < KB; ++ks) {
+            fa[ks] = *reinterpret_cast<const bf16x8 *>(qp + 16 * (k0 + ks));
+            fb[ks] = *reinterpret_cast<const bf16x8 *>(gp + 16 * (k0 + ks));
+          }
+#pragma unroll
+          for (int ks = 0; ks < KB; ++ks) {
+            s = mfma32(fa[ks], kf[k0 + ks], s);
+            dp = mfma32(fb[ks], vf[k0 + ks], dp);
+          }
+        }
         float p[16], ds[16];
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {

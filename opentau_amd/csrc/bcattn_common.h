@@ -138,6 +138,20 @@ __device__ __forceinline__ void tr_store_4x8(bf16_t *tile, int d0, int kg, bf16x
   }
 }
 
+// Row j of an operand that comes in two segments (n0 rows, then the rest).
+__device__ __forceinline__ const bf16_t *seg_row(const bf16_t *b0, int64_t s0, const bf16_t *b1,
+                                                 int64_t s1, int n0, int j) {
+  return j < n0 ? b0 + (int64_t)j * s0 : b1 + (int64_t)(j - n0) * s1;
+}
+
+// Loads are issued unconditionally from a clamped (always valid) address and
+// zeroed afterwards, so that a tile's loads are all in flight together instead
+// of each sitting in its own branch.
+__device__ __forceinline__ bf16x8 keep_if(bool ok, bf16x8 v) {
+  const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+  return ok ? v : z;
+}
+
 // ---------------------------------------------------------------------------
 // Kernel argument blocks (device pointers already offset to element 0).
 // ---------------------------------------------------------------------------

@@ -19,28 +19,31 @@ namespace bcattn {
 // writes its unnormalised fp32 partial (O, running max, sum) and
 // `fwd_combine_kernel` merges them.  This is what lets a handful of
 // (batch, kv head) problems with few query rows fill the chip.
-template <int D, bool SPLIT>
-__global__ __launch_bounds__(256) void fwd_bf16_kernel(const FwdArgs a, const SplitArgs sp) {
+template <int D, int NW, bool SPLIT>
+__global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, const SplitArgs sp) {
   constexpr int BN = 64;
+  constexpr int NT = 64 * NW;   // threads
+  constexpr int BM = 32 * NW;   // packed query rows per workgroup
   constexpr int KP = RowTile<D>::kPitch;
   constexpr int DK = D / 16;   // contraction steps of K Q^T
   constexpr int DB = D / 32;   // 32-row blocks of O^T
   constexpr int CPR = D / 8;   // 16-byte chunks per row
-  constexpr int KCH = (BN * CPR) / 256;
+  constexpr int KCH = (BN * CPR) / NT;
   constexpr int VUNITS = 16 * CPR;  // 4x8 transposition units per V tile
-  constexpr int VUN = (VUNITS + 255) / 256;
+  constexpr int VUN = (VUNITS + NT - 1) / NT;
+  static_assert((BN * CPR) % NT == 0, "K tile must divide over the threads");
 
   __shared__ __align__(16) bf16_t Ks[BN * KP];
   __shared__ __align__(16) bf16_t Vt[D * BN];
   __shared__ __align__(16) int kb_s[BN];
-  __shared__ int red_s[8];
+  __shared__ int red_s[2 * NW];
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
 
   const int R = a.G * a.Sq;
-  const int ntile_r = (R + 127) / 128;
+  const int ntile_r = (R + BM - 1) / BM;
   int bid = blockIdx.x;
   const int tile = bid % ntile_r;
   bid /= ntile_r;
@@ -50,7 +53,7 @@ __global__ __launch_bounds__(256) void fwd_bf16_kernel(const FwdArgs a, const Sp
   const int b = bid / a.Hkv;
 
   // ---- this lane's query row ------------------------------------------------
-  const int r = tile * 128 + wave * 32 + n;
+  const int r = tile * BM + wave * 32 + n;
   const bool rowok = r < R;
   const int rr = rowok ? r : R - 1;
   const int g = rr / a.Sq;
@@ -72,23 +75,29 @@ __global__ __launch_bounds__(256) void fwd_bf16_kernel(const FwdArgs a, const Sp
   const int any_w = wave_max_i(qv ? 1 : 0);
   if (lane == 0) {
     red_s[wave] = qmax_w;
-    red_s[4 + wave] = any_w;
+    red_s[NW + wave] = any_w;
   }
   __syncthreads();
-  const int qmax_g = max(max(red_s[0], red_s[1]), max(red_s[2], red_s[3]));
-  const int any_g = red_s[4] | red_s[5] | red_s[6] | red_s[7];
+  int qmax_g = kIntMin, any_g = 0;
+#pragma unroll
+  for (int x = 0; x < NW; ++x) {
+    qmax_g = max(qmax_g, red_s[x]);
+    any_g |= red_s[NW + x];
+  }
 
   const int Sk = a.Sk;
   const int nt_all = (Sk + BN - 1) / BN;
   const int t_first = SPLIT ? split * sp.tiles_per_split : 0;
   const int nt = !any_g ? 0 : (SPLIT ? min(nt_all, t_first + sp.tiles_per_split) : nt_all);
-  const tile_summary_t *ksum = a.ksum + (int64_t)b * ((Sk + BN - 1) / BN);
+  const tile_summary_t *ksum = a.ksum + (int64_t)b * nt_all;
 
   const bf16_t *k0b = reinterpret_cast<const bf16_t *>(a.k0.ptr) + b * a.k0.sb + hk * a.k0.sh;
   const bf16_t *v0b = reinterpret_cast<const bf16_t *>(a.v0.ptr) + b * a.v0.sb + hk * a.v0.sh;
   const bf16_t *k1b = reinterpret_cast<const bf16_t *>(a.k1.ptr) + b * a.k1.sb + hk * a.k1.sh;
   const bf16_t *v1b = reinterpret_cast<const bf16_t *>(a.v1.ptr) + b * a.v1.sb + hk * a.v1.sh;
   const int Sk0 = a.Sk0;
+  const int32_t *kblk_b = a.k_blk + (int64_t)b * Sk;
+  const uint8_t *kval_b = a.k_valid + (int64_t)b * Sk;
 
   bf16x8 kreg[KCH];
   bf16x8 vreg[VUN][4];
@@ -99,53 +108,48 @@ __global__ __launch_bounds__(256) void fwd_bf16_kernel(const FwdArgs a, const Sp
     return t;
   };
 
+  // Global loads of one tile into registers (consumed by stage() one iteration later).
   auto prefetch = [&](int t) {
     const int j0 = t * BN;
 #pragma unroll
     for (int it = 0; it < KCH; ++it) {
-      const int c = tid + 256 * it;
+      const int c = tid + NT * it;
       const int row = c / CPR, col = c % CPR;
-      const int j = j0 + row;
-      bf16x8 val = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (j < Sk) {
-        const bf16_t *p = (j < Sk0) ? k0b + (int64_t)j * a.k0.ss : k1b + (int64_t)(j - Sk0) * a.k1.ss;
-        val = *reinterpret_cast<const bf16x8 *>(p + col * 8);
-      }
-      kreg[it] = val;
+      const int j = j0 + row, jc = min(j, Sk - 1);
+      const bf16x8 val =
+          *reinterpret_cast<const bf16x8 *>(seg_row(k0b, a.k0.ss, k1b, a.k1.ss, Sk0, jc) + col * 8);
+      kreg[it] = keep_if(j < Sk, val);
     }
 #pragma unroll
     for (int it = 0; it < VUN; ++it) {
-      const int u = tid + 256 * it;
+      const int u = min(tid + NT * it, VUNITS - 1);
       const int dch = u % CPR, kg = u / CPR;
 #pragma unroll
       for (int x = 0; x < 4; ++x) {
-        const int j = j0 + 4 * kg + x;
-        bf16x8 val = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (u < VUNITS && j < Sk) {
-          const bf16_t *p =
-              (j < Sk0) ? v0b + (int64_t)j * a.v0.ss : v1b + (int64_t)(j - Sk0) * a.v1.ss;
-          val = *reinterpret_cast<const bf16x8 *>(p + dch * 8);
-        }
-        vreg[it][x] = val;
+        const int j = j0 + 4 * kg + x, jc = min(j, Sk - 1);
+        const bf16x8 val =
+            *reinterpret_cast<const bf16x8 *>(seg_row(v0b, a.v0.ss, v1b, a.v1.ss, Sk0, jc) + dch * 8);
+        vreg[it][x] = keep_if(j < Sk, val);
       }
     }
-    if (tid < BN) {
-      const int j = j0 + tid;
-      kbreg = kIntMax;
-      if (j < Sk && a.k_valid[(int64_t)b * Sk + j]) kbreg = a.k_blk[(int64_t)b * Sk + j];
+    {
+      const int j = j0 + (tid & (BN - 1)), jc = min(j, Sk - 1);
+      const int id = kblk_b[jc];
+      const int ok = kval_b[jc];
+      kbreg = (j < Sk && ok != 0) ? id : kIntMax;
     }
   };
 
   auto stage = [&]() {
 #pragma unroll
     for (int it = 0; it < KCH; ++it) {
-      const int c = tid + 256 * it;
+      const int c = tid + NT * it;
       const int row = c / CPR, col = c % CPR;
       *reinterpret_cast<bf16x8 *>(Ks + row * KP + col * 8) = kreg[it];
     }
 #pragma unroll
     for (int it = 0; it < VUN; ++it) {
-      const int u = tid + 256 * it;
+      const int u = tid + NT * it;
       const int dch = u % CPR, kg = u / CPR;
       if (u < VUNITS) tr_store_4x8(Vt, 8 * dch, kg, vreg[it][0], vreg[it][1], vreg[it][2], vreg[it][3]);
     }
@@ -178,11 +182,11 @@ __global__ __launch_bounds__(256) void fwd_bf16_kernel(const FwdArgs a, const Sp
 #pragma unroll
         for (int x = 0; x < 16; ++x) s[mb][x] = 0.f;
         const bf16_t *kp = Ks + (32 * mb + n) * KP + 8 * hh;
+        bf16x8 ka[DK];
 #pragma unroll
-        for (int ks = 0; ks < DK; ++ks) {
-          const bf16x8 ka = *reinterpret_cast<const bf16x8 *>(kp + 16 * ks);
-          s[mb] = mfma32(ka, qf[ks], s[mb]);
-        }
+        for (int ks = 0; ks < DK; ++ks) ka[ks] = *reinterpret_cast<const bf16x8 *>(kp + 16 * ks);
+#pragma unroll
+        for (int ks = 0; ks < DK; ++ks) s[mb] = mfma32(ka[ks], qf[ks], s[mb]);
       }
       const bool needmask = !(sm.z != 0 && sm.y <= qmin_w);
       if (needmask) {
@@ -228,11 +232,12 @@ __global__ __launch_bounds__(256) void fwd_bf16_kernel(const FwdArgs a, const Sp
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         const int d = 32 * db + n;
+        bf16x8 va[4];
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-          const bf16x8 va = *reinterpret_cast<const bf16x8 *>(Vt + tr_read_off(d, kk, hh));
-          o[db] = mfma32(va, pb[kk], o[db]);
-        }
+        for (int kk = 0; kk < 4; ++kk)
+          va[kk] = *reinterpret_cast<const bf16x8 *>(Vt + tr_read_off(d, kk, hh));
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) o[db] = mfma32(va[kk], pb[kk], o[db]);
       }
     }
     __syncthreads();
@@ -326,18 +331,20 @@ __global__ __launch_bounds__(256) void fwd_combine_kernel(const FwdArgs a, const
 
 int launch_fwd_bf16(const FwdArgs &a, int D, hipStream_t st) {
   const int R = a.G * a.Sq;
-  const int ntile_r = (R + 127) / 128;
-  const dim3 grid((unsigned)(ntile_r * a.Hkv * a.B)), block(256);
   const SplitArgs sp{nullptr, nullptr, 1, 0};
+  auto grid = [&](int bm) { return dim3((unsigned)(((R + bm - 1) / bm) * a.Hkv * a.B)); };
   switch (D) {
     case 64:
-      hipLaunchKernelGGL((fwd_bf16_kernel<64, false>), grid, block, 0, st, a, sp);
+      hipLaunchKernelGGL((fwd_bf16_kernel<64, 4, false>), grid(128), dim3(256), 0, st, a, sp);
       break;
     case 128:
-      hipLaunchKernelGGL((fwd_bf16_kernel<128, false>), grid, block, 0, st, a, sp);
+      if (R >= 1024)
+        hipLaunchKernelGGL((fwd_bf16_kernel<128, 8, false>), grid(256), dim3(512), 0, st, a, sp);
+      else
+        hipLaunchKernelGGL((fwd_bf16_kernel<128, 4, false>), grid(128), dim3(256), 0, st, a, sp);
       break;
     case 256:
-      hipLaunchKernelGGL((fwd_bf16_kernel<256, false>), grid, block, 0, st, a, sp);
+      hipLaunchKernelGGL((fwd_bf16_kernel<256, 4, false>), grid(128), dim3(256), 0, st, a, sp);
       break;
     default:
       return BCATTN_ERR_UNSUPPORTED;
@@ -371,7 +378,7 @@ template <int D>
 static int launch_split(const FwdArgs &a, const SplitArgs &sp, hipStream_t st) {
   const int R = a.G * a.Sq;
   const int ntile_r = (R + 127) / 128;
-  hipLaunchKernelGGL((fwd_bf16_kernel<D, true>), dim3((unsigned)(ntile_r * sp.nsplit * a.Hkv * a.B)),
+  hipLaunchKernelGGL((fwd_bf16_kernel<D, 4, true>), dim3((unsigned)(ntile_r * sp.nsplit * a.Hkv * a.B)),
                      dim3(256), 0, st, a, sp);
   constexpr int RPB = 256 / (D / 4);
   const int64_t rows = (int64_t)a.B * a.Hkv * R;

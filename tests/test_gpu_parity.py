@@ -386,8 +386,9 @@ def test_autograd_op_matches_raw_backward():
     vc, vn = v.detach()[:, :40].clone().requires_grad_(True), v.detach()[:, 40:].clone().requires_grad_(True)
     q2 = q.detach().clone().requires_grad_(True)
     fa.flash_attn_blockmask_kvcache(q2, kc, vc, kn, vn, *ids, d**-0.5).backward(go)
-    assert torch.equal(torch.cat([kc.grad, kn.grad], 1), dk) and torch.equal(torch.cat([vc.grad, vn.grad], 1), dv)
-    assert torch.equal(q2.grad, dq)
+    # (the cached forward may split the key axis, so its saved O / LSE differ in the last bit)
+    for got, ref in ((torch.cat([kc.grad, kn.grad], 1), dk), (torch.cat([vc.grad, vn.grad], 1), dv), (q2.grad, dq)):
+        assert rel_l2(got.float(), ref.float()) <= 5e-3
 
 
 # --------------------------------------------------------------------------- #
