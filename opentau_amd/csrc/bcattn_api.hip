@@ -17,37 +17,56 @@ static int fail(int code, const char *fmt, ...) {
   return code;
 }
 
-// ---- key / query tile summaries ------------------------------------------------
-__global__ __launch_bounds__(64) void summary_kernel(const int32_t *blk, const uint8_t *valid, int S,
-                                                     int ntile, tile_summary_t *out) {
+// ---- tile summaries and merged ids -----------------------------------------------
+// The sequence is cut into 64-wide tiles that never straddle its two segments
+// (n0 rows, then S - n0): tiles [0, nt0) cover segment 0, the rest segment 1,
+// each segment padded at its end.  Per tile the kernel writes the summary
+// (min / max id over valid positions, all-valid flag, count) and, per slot, the
+// id with `fill` in place of invalid or padding positions, so that the
+// attention kernels need one compare per pair and one 256-byte load per tile.
+__global__ __launch_bounds__(64) void summary_kernel(const int32_t *blk, const uint8_t *valid, int n0,
+                                                     int S, int nt0, int ntile, int fill,
+                                                     tile_summary_t *sum, int32_t *merged) {
   const int t = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
-  const int j = t * kSumTile + lane;
-  const bool ok = j < S && valid[(int64_t)b * S + j] != 0;
+  const int seg = t >= nt0;
+  const int pos = (seg ? t - nt0 : t) * kSumTile + lane;  // position inside the segment
+  const int len = seg ? S - n0 : n0;
+  const int j = (seg ? n0 : 0) + pos;
+  const bool ok = pos < len && valid[(int64_t)b * S + j] != 0;
   const int id = ok ? blk[(int64_t)b * S + j] : 0;
   const int mn = wave_min_i(ok ? id : kIntMax);
   const int mx = wave_max_i(ok ? id : kIntMin);
   const int cnt = wave_sum_i(ok ? 1 : 0);
+  merged[((int64_t)b * ntile + t) * kSumTile + lane] = ok ? id : fill;
   if (lane == 0) {
     tile_summary_t s;
     s.x = mn;
     s.y = mx;
     s.z = cnt == kSumTile ? 1 : 0;
     s.w = cnt;
-    out[(int64_t)b * ntile + t] = s;
+    sum[(int64_t)b * ntile + t] = s;
   }
 }
 
-int launch_summary(const int32_t *blk, const uint8_t *valid, int B, int S, tile_summary_t *out,
-                   hipStream_t st) {
-  const int ntile = (S + kSumTile - 1) / kSumTile;
-  hipLaunchKernelGGL(summary_kernel, dim3(ntile, B), dim3(64), 0, st, blk, valid, S, ntile, out);
+static int ntiles(int n0, int S) { return (n0 + kSumTile - 1) / kSumTile + (S - n0 + kSumTile - 1) / kSumTile; }
+
+int launch_summary(const int32_t *blk, const uint8_t *valid, int B, int n0, int S, int fill,
+                   tile_summary_t *sum, int32_t *merged, hipStream_t st) {
+  const int nt0 = (n0 + kSumTile - 1) / kSumTile;
+  const int nt = ntiles(n0, S);
+  hipLaunchKernelGGL(summary_kernel, dim3(nt, B), dim3(64), 0, st, blk, valid, n0, S, nt0, nt, fill, sum,
+                     merged);
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
 }
 
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
-static size_t summary_bytes(int B, int S) {
-  return align256((size_t)B * ((S + kSumTile - 1) / kSumTile) * sizeof(tile_summary_t));
+static size_t summary_bytes(int B, int n0, int S) {
+  return align256((size_t)B * ntiles(n0, S) * sizeof(tile_summary_t));
 }
+static size_t merged_bytes(int B, int n0, int S) {
+  return align256((size_t)B * ntiles(n0, S) * kSumTile * sizeof(int32_t));
+}
+static int pad64(int s) { return (s + 63) / 64 * 64; }
 
 static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
@@ -59,6 +78,20 @@ static int check_tensor(const char *name, const bcattn_tensor &t, int vec, bool 
   if (!aligned16(t.ptr)) return fail(BCATTN_ERR_INVALID, "%s: pointer not 16-byte aligned", name);
   if (t.stride_b % vec || t.stride_s % vec || t.stride_h % vec)
     return fail(BCATTN_ERR_INVALID, "%s: strides must be multiples of %d elements", name, vec);
+  if (t.stride_b < 0 || t.stride_s <= 0 || t.stride_h < 0)
+    return fail(BCATTN_ERR_INVALID, "%s: strides must be non-negative (sequence stride positive)", name);
+  return BCATTN_OK;
+}
+
+// The MFMA kernels address a (batch, head) slab of an operand through a 32-bit
+// buffer descriptor: rows * stride * 2 bytes must stay below 2^31.
+static int check_span(const char *name, const bcattn_tensor &t, int rows, int D, int dtype) {
+  if (dtype != BCATTN_BF16 || t.ptr == nullptr) return BCATTN_OK;
+  if (t.stride_s < D) return fail(BCATTN_ERR_INVALID, "%s: sequence stride smaller than head_dim", name);
+  const int64_t bytes = ((int64_t)(rows - 1) * t.stride_s + D) * 2;
+  if (bytes >= ((int64_t)1 << 31))
+    return fail(BCATTN_ERR_UNSUPPORTED, "%s: one (batch, head) slab spans %lld bytes; the limit is 2 GiB", name,
+                (long long)bytes);
   return BCATTN_OK;
 }
 
@@ -77,6 +110,8 @@ static int check_common(int B, int Sq, int Sk, int H, int Hkv, int D, int dtype,
     return fail(BCATTN_ERR_UNSUPPORTED, "dtype %d not supported (0 = fp32, 1 = bf16)", dtype);
   }
   if ((int64_t)(H / Hkv) * Sq > 0x3fffffff) return fail(BCATTN_ERR_INVALID, "G*Sq too large");
+  if ((int64_t)B * H * pad64(Sq) * 4 >= ((int64_t)1 << 31) || (int64_t)B * (Sk + 128) * 4 >= ((int64_t)1 << 31))
+    return fail(BCATTN_ERR_UNSUPPORTED, "B*H*Sq too large for the 32-bit statistics buffers");
   return BCATTN_OK;
 }
 
@@ -96,6 +131,12 @@ static int check_fwd(const bcattn_fwd_params *p) {
   if ((rc = check_tensor("k1", p->k1, vec, p->Sk1 > 0))) return rc;
   if ((rc = check_tensor("v1", p->v1, vec, p->Sk1 > 0))) return rc;
   if ((rc = check_tensor("o", p->o, vec, true))) return rc;
+  if (p->Sk0 > 0 && ((rc = check_span("k", p->k, p->Sk0, p->D, p->dtype)) ||
+                     (rc = check_span("v", p->v, p->Sk0, p->D, p->dtype))))
+    return rc;
+  if (p->Sk1 > 0 && ((rc = check_span("k1", p->k1, p->Sk1, p->D, p->dtype)) ||
+                     (rc = check_span("v1", p->v1, p->Sk1, p->D, p->dtype))))
+    return rc;
   if (!p->q_blk || !p->k_blk || !p->q_valid || !p->k_valid)
     return fail(BCATTN_ERR_INVALID, "null block-id / valid pointer");
   return BCATTN_OK;
@@ -118,6 +159,7 @@ static FwdArgs fwd_args(const bcattn_fwd_params *p) {
   a.q_valid = p->q_valid;
   a.k_valid = p->k_valid;
   a.ksum = nullptr;
+  a.kbm = nullptr;
   a.B = p->B;
   a.Sq = p->Sq;
   a.Sk0 = p->Sk0;
@@ -127,6 +169,21 @@ static FwdArgs fwd_args(const bcattn_fwd_params *p) {
   a.G = p->H / p->Hkv;
   a.scale = p->scale;
   return a;
+}
+
+// Forward workspace: [tile summaries][merged key ids]( [split partials] ).
+static int fwd_prepare(const bcattn_fwd_params *p, FwdArgs &a, char *&ws, hipStream_t st) {
+  tile_summary_t *ks = reinterpret_cast<tile_summary_t *>(ws);
+  ws += summary_bytes(a.B, a.Sk0, a.Sk);
+  int32_t *km = reinterpret_cast<int32_t *>(ws);
+  ws += merged_bytes(a.B, a.Sk0, a.Sk);
+  if (!p->summary_ready) {
+    const int rc = launch_summary(p->k_blk, p->k_valid, a.B, a.Sk0, a.Sk, kIntMax, ks, km, st);
+    if (rc) return fail(rc, "summary launch failed: %s", hipGetErrorString(hipGetLastError()));
+  }
+  a.ksum = ks;
+  a.kbm = km;
+  return BCATTN_OK;
 }
 
 }  // namespace bcattn
@@ -141,20 +198,21 @@ const char *bcattn_last_error(void) { return g_err; }
 
 size_t bcattn_fwd_workspace_bytes(const bcattn_fwd_params *p) {
   if (p == nullptr || p->B <= 0) return 0;
-  return summary_bytes(p->B, p->Sk0 + p->Sk1);
+  return summary_bytes(p->B, p->Sk0, p->Sk0 + p->Sk1) + merged_bytes(p->B, p->Sk0, p->Sk0 + p->Sk1);
 }
 
 size_t bcattn_fwd_kvcache_workspace_bytes(const bcattn_fwd_params *p) {
   if (p == nullptr || p->B <= 0) return 0;
   int ns = 0;
-  return summary_bytes(p->B, p->Sk0 + p->Sk1) +
-         kvcache_workspace_bytes(p->B, p->Sq, p->Sk0 + p->Sk1, p->H, p->Hkv, p->D, &ns);
+  return bcattn_fwd_workspace_bytes(p) +
+         kvcache_workspace_bytes(p->B, p->Sq, p->Sk0, p->Sk0 + p->Sk1, p->H, p->Hkv, p->D, &ns);
 }
 
 size_t bcattn_bwd_workspace_bytes(const bcattn_bwd_params *p) {
   if (p == nullptr || p->B <= 0) return 0;
-  return summary_bytes(p->B, p->Sk) + summary_bytes(p->B, p->Sq) +
-         align256((size_t)p->B * p->H * p->Sq * sizeof(float));
+  return summary_bytes(p->B, p->Sk, p->Sk) + merged_bytes(p->B, p->Sk, p->Sk) +
+         summary_bytes(p->B, p->Sq, p->Sq) + merged_bytes(p->B, p->Sq, p->Sq) +
+         2 * align256((size_t)p->B * p->H * pad64(p->Sq) * sizeof(float));
 }
 
 int bcattn_fwd(const bcattn_fwd_params *p, void *stream) {
@@ -167,12 +225,8 @@ int bcattn_fwd(const bcattn_fwd_params *p, void *stream) {
                 need, p->workspace ? p->workspace_bytes : (size_t)0);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   FwdArgs a = fwd_args(p);
-  tile_summary_t *ks = reinterpret_cast<tile_summary_t *>(p->workspace);
-  if (!p->summary_ready) {
-    rc = launch_summary(p->k_blk, p->k_valid, a.B, a.Sk, ks, st);
-    if (rc) return fail(rc, "summary launch failed: %s", hipGetErrorString(hipGetLastError()));
-  }
-  a.ksum = ks;
+  char *ws = reinterpret_cast<char *>(p->workspace);
+  if ((rc = fwd_prepare(p, a, ws, st))) return rc;
   rc = p->dtype == BCATTN_BF16 ? launch_fwd_bf16(a, p->D, st) : launch_fwd_f32(a, p->D, st);
   if (rc) return fail(rc, "forward launch failed (D=%d dtype=%d)", p->D, p->dtype);
   return BCATTN_OK;
@@ -190,19 +244,13 @@ int bcattn_fwd_kvcache(const bcattn_fwd_params *p, void *stream) {
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   FwdArgs a = fwd_args(p);
   char *ws = reinterpret_cast<char *>(p->workspace);
-  tile_summary_t *ks = reinterpret_cast<tile_summary_t *>(ws);
-  if (!p->summary_ready) {
-    rc = launch_summary(p->k_blk, p->k_valid, a.B, a.Sk, ks, st);
-    if (rc) return fail(rc, "summary launch failed: %s", hipGetErrorString(hipGetLastError()));
-  }
-  a.ksum = ks;
-  ws += summary_bytes(a.B, a.Sk);
+  if ((rc = fwd_prepare(p, a, ws, st))) return rc;
   SplitArgs s;
-  const size_t part = kvcache_workspace_bytes(a.B, a.Sq, a.Sk, a.H, a.Hkv, p->D, &s.nsplit);
+  s.tiles_per_split = 0;
+  kvcache_workspace_bytes(a.B, a.Sq, a.Sk0, a.Sk, a.H, a.Hkv, p->D, &s.nsplit);
   const size_t R = (size_t)a.G * a.Sq;
   s.part_o = reinterpret_cast<float *>(ws);
   s.part_ml = s.part_o + (size_t)a.B * a.Hkv * s.nsplit * R * p->D;
-  (void)part;
   rc = launch_fwd_kvcache_bf16(a, s, p->D, st);
   if (rc) return fail(rc, "kvcache forward launch failed (D=%d)", p->D);
   return BCATTN_OK;
@@ -216,10 +264,12 @@ int bcattn_bwd(const bcattn_bwd_params *p, void *stream) {
   const struct {
     const char *n;
     const bcattn_tensor *t;
-  } ts[] = {{"q", &p->q},   {"k", &p->k},   {"v", &p->v},   {"o", &p->o},
-            {"d_o", &p->d_o}, {"dq", &p->dq}, {"dk", &p->dk}, {"dv", &p->dv}};
+    int rows;
+  } ts[] = {{"q", &p->q, p->Sq},   {"k", &p->k, p->Sk},   {"v", &p->v, p->Sk},   {"o", &p->o, p->Sq},
+            {"d_o", &p->d_o, p->Sq}, {"dq", &p->dq, p->Sq}, {"dk", &p->dk, p->Sk}, {"dv", &p->dv, p->Sk}};
   for (auto &e : ts)
-    if ((rc = check_tensor(e.n, *e.t, vec, true))) return rc;
+    if ((rc = check_tensor(e.n, *e.t, vec, true)) || (rc = check_span(e.n, *e.t, e.rows, p->D, p->dtype)))
+      return rc;
   if (!p->lse || !p->q_blk || !p->k_blk || !p->q_valid || !p->k_valid)
     return fail(BCATTN_ERR_INVALID, "null lse / block-id / valid pointer");
   if (p->B == 0) return BCATTN_OK;
@@ -243,20 +293,27 @@ int bcattn_bwd(const bcattn_bwd_params *p, void *stream) {
   a.lse = p->lse;
   a.q_blk = p->q_blk, a.k_blk = p->k_blk, a.q_valid = p->q_valid, a.k_valid = p->k_valid;
   a.B = p->B, a.Sq = p->Sq, a.Sk = p->Sk, a.H = p->H, a.Hkv = p->Hkv, a.G = p->H / p->Hkv;
+  a.Sq_pad = pad64(p->Sq);
   a.scale = p->scale;
   a.stages = p->stages & (BCATTN_BWD_DELTA | BCATTN_BWD_DQ | BCATTN_BWD_DKV);
   if (a.stages == 0) a.stages = BCATTN_BWD_DELTA | BCATTN_BWD_DQ | BCATTN_BWD_DKV;
+  // Backward workspace: [key summaries][key ids][query summaries][query ids][delta][log2e*LSE].
   char *ws = reinterpret_cast<char *>(p->workspace);
   tile_summary_t *ks = reinterpret_cast<tile_summary_t *>(ws);
-  ws += summary_bytes(a.B, a.Sk);
+  ws += summary_bytes(a.B, a.Sk, a.Sk);
+  int32_t *km = reinterpret_cast<int32_t *>(ws);
+  ws += merged_bytes(a.B, a.Sk, a.Sk);
   tile_summary_t *qs = reinterpret_cast<tile_summary_t *>(ws);
-  ws += summary_bytes(a.B, a.Sq);
+  ws += summary_bytes(a.B, a.Sq, a.Sq);
+  int32_t *qm = reinterpret_cast<int32_t *>(ws);
+  ws += merged_bytes(a.B, a.Sq, a.Sq);
   a.delta = reinterpret_cast<float *>(ws);
-  a.ksum = ks;
-  a.qsum = qs;
+  ws += align256((size_t)a.B * a.H * a.Sq_pad * sizeof(float));
+  a.lse2 = reinterpret_cast<float *>(ws);
+  a.ksum = ks, a.qsum = qs, a.kbm = km, a.qbm = qm;
   if (!p->summary_ready &&
-      ((rc = launch_summary(p->k_blk, p->k_valid, a.B, a.Sk, ks, st)) ||
-       (rc = launch_summary(p->q_blk, p->q_valid, a.B, a.Sq, qs, st))))
+      ((rc = launch_summary(p->k_blk, p->k_valid, a.B, a.Sk, a.Sk, kIntMax, ks, km, st)) ||
+       (rc = launch_summary(p->q_blk, p->q_valid, a.B, a.Sq, a.Sq, kIntMin, qs, qm, st))))
     return fail(rc, "summary launch failed");
   rc = p->dtype == BCATTN_BF16 ? launch_bwd_bf16(a, p->D, st) : launch_bwd_f32(a, p->D, st);
   if (rc) return fail(rc, "backward launch failed (D=%d dtype=%d)", p->D, p->dtype);

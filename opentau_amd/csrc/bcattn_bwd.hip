@@ -1,8 +1,10 @@
 // Block-causal attention backward, bf16 in / fp32 accumulate, gfx950 MFMA.
 //
 // Three kernels, no atomics, so gradients are bit-repeatable:
-//   delta   delta[b,h,i] = sum_d O*dO
-//   dQ      a workgroup owns 128 packed query rows and streams key tiles;
+//   prep    delta[b,h,i] = sum_d O*dO, and log2e*LSE (+inf on rows that take no
+//           part), both padded to whole 64-row tiles so that the dK/dV kernel can
+//           pull them into LDS with one buffer load
+//   dQ      a workgroup owns 32*NW packed query rows and streams key tiles;
 //           dQ^T = K^T dS^T with dS^T = P^T o (dP^T - delta), all keys x queries
 //   dK/dV   a workgroup owns 128 keys of one kv head and streams the query tiles
 //           of every query head of its group, so the sum over the GQA group
@@ -10,119 +12,76 @@
 // P is recomputed from the saved log-sum-exp: P = exp2(scale*log2e*S - log2e*LSE).
 //
 // As in the forward, the 32x32 accumulator of the first product is already the B
-// operand of the second, so P / dS never leave registers; the operand that must
-// be contracted over the sequence axis (K^T, Q^T, dO^T) is kept in LDS as a
-// transposed tile next to the row tile.
-#include "bcattn_common.h"
+// operand of the second, so P / dS never leave registers.  Streamed tiles go
+// from global memory straight into swizzled LDS tiles (no registers, no LDS
+// stores), double buffered; the operand that must be contracted over the
+// sequence axis (K^T, Q^T, dO^T) is read from the same row-major tile with the
+// transposing LDS read.
+#include "bcattn_tiles.h"
 
 namespace bcattn {
 
-// ---- tile movers -------------------------------------------------------------
-// A 64 x D tile is moved as 16*(D/8) units of 4 rows x 8 columns: four 16-byte
-// global loads per unit, then four 16-byte row stores and/or eight 8-byte
-// transposed stores.
+// ---- prep: delta and scaled LSE, padded -------------------------------------------
 template <int D>
-struct TileUnits {
-  static constexpr int CPR = D / 8;
-  static constexpr int UNITS = 16 * CPR;
-  static constexpr int NU = (UNITS + 255) / 256;
-};
-
-template <int D>
-__device__ __forceinline__ void load_units(bf16x8 (&reg)[TileUnits<D>::NU][4], const bf16_t *base,
-                                           int64_t row_stride, int row0, int nrows, int tid) {
-  using T = TileUnits<D>;
-#pragma unroll
-  for (int it = 0; it < T::NU; ++it) {
-    const int u = min(tid + 256 * it, T::UNITS - 1);
-    const int dch = u % T::CPR, kg = u / T::CPR;
-#pragma unroll
-    for (int x = 0; x < 4; ++x) {
-      const int row = row0 + 4 * kg + x, rc = min(row, nrows - 1);
-      const bf16x8 val = *reinterpret_cast<const bf16x8 *>(base + (int64_t)rc * row_stride + dch * 8);
-      reg[it][x] = keep_if(row < nrows, val);
-    }
-  }
-}
-
-template <int D, bool ROWS, bool TRANS>
-__device__ __forceinline__ void store_units(const bf16x8 (&reg)[TileUnits<D>::NU][4], bf16_t *rows,
-                                            bf16_t *trans, int tid) {
-  using T = TileUnits<D>;
-  constexpr int KP = RowTile<D>::kPitch;
-#pragma unroll
-  for (int it = 0; it < T::NU; ++it) {
-    const int u = tid + 256 * it;
-    const int dch = u % T::CPR, kg = u / T::CPR;
-    if (u < T::UNITS) {
-      if (ROWS) {
-#pragma unroll
-        for (int x = 0; x < 4; ++x)
-          *reinterpret_cast<bf16x8 *>(rows + (4 * kg + x) * KP + dch * 8) = reg[it][x];
-      }
-      if (TRANS) tr_store_4x8(trans, 8 * dch, kg, reg[it][0], reg[it][1], reg[it][2], reg[it][3]);
-    }
-  }
-}
-
-// ---- delta ---------------------------------------------------------------------
-template <int D>
-__global__ __launch_bounds__(256) void bwd_delta_kernel(const BwdArgs a) {
+__global__ __launch_bounds__(256) void bwd_prep_kernel(const BwdArgs a) {
   constexpr int LPR = D / 8;
   constexpr int RPB = 256 / LPR;
-  const int64_t total = (int64_t)a.B * a.Sq * a.H;
+  const int Sqp = a.Sq_pad;
+  const int64_t total = (int64_t)a.B * a.H * Sqp;  // (b, h, i) with i fastest
   const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
   const int c = threadIdx.x % LPR;
   float acc = 0.f;
   int h = 0, i = 0, b = 0;
+  bool real = false;
   if (row < total) {
-    h = (int)(row % a.H);
-    i = (int)((row / a.H) % a.Sq);
-    b = (int)(row / ((int64_t)a.H * a.Sq));
-    const bf16x8 ov = *reinterpret_cast<const bf16x8 *>(
-        reinterpret_cast<const bf16_t *>(a.o.ptr) + b * a.o.sb + (int64_t)i * a.o.ss + h * a.o.sh + 8 * c);
-    const bf16x8 gv = *reinterpret_cast<const bf16x8 *>(reinterpret_cast<const bf16_t *>(a.d_o.ptr) +
-                                                        b * a.d_o.sb + (int64_t)i * a.d_o.ss +
-                                                        h * a.d_o.sh + 8 * c);
+    i = (int)(row % Sqp);
+    h = (int)((row / Sqp) % a.H);
+    b = (int)(row / ((int64_t)Sqp * a.H));
+    real = i < a.Sq;
+    if (real) {
+      const bf16x8 ov = *reinterpret_cast<const bf16x8 *>(reinterpret_cast<const bf16_t *>(a.o.ptr) +
+                                                          b * a.o.sb + (int64_t)i * a.o.ss + h * a.o.sh + 8 * c);
+      const bf16x8 gv = *reinterpret_cast<const bf16x8 *>(reinterpret_cast<const bf16_t *>(a.d_o.ptr) +
+                                                          b * a.d_o.sb + (int64_t)i * a.d_o.ss +
+                                                          h * a.d_o.sh + 8 * c);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc += (float)ov[e] * (float)gv[e];
+      for (int e = 0; e < 8; ++e) acc += (float)ov[e] * (float)gv[e];
+    }
   }
 #pragma unroll
   for (int o = LPR / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-  if (row < total && c == 0) a.delta[((int64_t)b * a.H + h) * a.Sq + i] = acc;
+  if (row < total && c == 0) {
+    const bool ok = real && a.q_valid[(int64_t)b * a.Sq + i] != 0;
+    a.delta[row] = ok ? acc : 0.f;
+    a.lse2[row] = ok ? a.lse[((int64_t)b * a.H + h) * a.Sq + i] * kLog2e : INFINITY;
+  }
 }
 
 // ---- dQ ------------------------------------------------------------------------
-template <int D, bool PF>
-__global__ __launch_bounds__(256) void bwd_dq_kernel(const BwdArgs a) {
-  constexpr int BN = 64;
-  constexpr int KP = RowTile<D>::kPitch;
-  constexpr int DK = D / 16;
-  constexpr int DB = D / 32;
-  constexpr int CPR = D / 8;
-  constexpr int VCH = (BN * CPR) / 256;
-  constexpr int NU = TileUnits<D>::NU;
+template <int D, int NW>
+__global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
+  using T = Tile<D>;
+  constexpr int NT = 64 * NW, BM = 32 * NW;
+  constexpr int DK = D / 16, DB = D / 32;
+  constexpr int STAGE = 2 * T::kBytes + 256;  // K tile, V tile, 64 key ids
 
-  extern __shared__ __align__(16) char smem_raw[];
-  bf16_t *Ks = reinterpret_cast<bf16_t *>(smem_raw);
-  bf16_t *Vs = Ks + BN * KP;
-  bf16_t *Kt = Vs + BN * KP;
-  int *kb_s = reinterpret_cast<int *>(Kt + D * BN);
-  int *red_s = kb_s + BN;
+  extern __shared__ __align__(1024) char smem[];
+  __shared__ int red_s[2 * NW];
 
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
 
   const int R = a.G * a.Sq;
-  const int ntile_r = (R + 127) / 128;
+  const int ntile_r = (R + BM - 1) / BM;
   int bid = blockIdx.x;
-  const int tile = bid % ntile_r;
+  const int tile = __builtin_amdgcn_readfirstlane(bid % ntile_r);
   bid /= ntile_r;
-  const int hk = bid % a.Hkv;
-  const int b = bid / a.Hkv;
+  // (division results live in vector registers; say that they are uniform)
+  const int hk = __builtin_amdgcn_readfirstlane(bid % a.Hkv);
+  const int b = __builtin_amdgcn_readfirstlane(bid / a.Hkv);
 
-  const int r = tile * 128 + wave * 32 + n;
+  const int r = tile * BM + wave * 32 + n;
   const bool rowok = r < R;
   const int rr = rowok ? r : R - 1;
   const int g = rr / a.Sq;
@@ -141,64 +100,62 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(const BwdArgs a) {
     qf[ks] = *reinterpret_cast<const bf16x8 *>(qptr + 16 * ks + 8 * hh);
     gof[ks] = *reinterpret_cast<const bf16x8 *>(gptr + 16 * ks + 8 * hh);
   }
-  const int64_t stat = ((int64_t)b * a.H + h) * a.Sq + i;
-  // Rows that take no part get +inf so that every probability comes out 0.
-  const float lse2 = qv ? a.lse[stat] * kLog2e : INFINITY;
-  const float delta = qv ? a.delta[stat] : 0.f;
+  const int64_t stat = ((int64_t)b * a.H + h) * a.Sq_pad + i;
+  const float lse2 = rowok ? a.lse2[stat] : INFINITY;  // +inf on rows that take no part
+  const float delta = rowok ? a.delta[stat] : 0.f;
 
   const int qmax_w = wave_max_i(qv ? qb : kIntMin);
   const int qmin_w = wave_min_i(qv ? qb : kIntMax);
   const int any_w = wave_max_i(qv ? 1 : 0);
   if (lane == 0) {
     red_s[wave] = qmax_w;
-    red_s[4 + wave] = any_w;
+    red_s[NW + wave] = any_w;
   }
   __syncthreads();
-  const int qmax_g = max(max(red_s[0], red_s[1]), max(red_s[2], red_s[3]));
-  const int any_g = red_s[4] | red_s[5] | red_s[6] | red_s[7];
+  int qmax_g = kIntMin, any_g = 0;
+#pragma unroll
+  for (int x = 0; x < NW; ++x) {
+    qmax_g = max(qmax_g, red_s[x]);
+    any_g |= red_s[NW + x];
+  }
 
   const int Sk = a.Sk;
-  const int nt = any_g ? (Sk + BN - 1) / BN : 0;
-  const tile_summary_t *ksum = a.ksum + (int64_t)b * ((Sk + BN - 1) / BN);
-  const bf16_t *kb_ = reinterpret_cast<const bf16_t *>(a.k.ptr) + b * a.k.sb + hk * a.k.sh;
-  const bf16_t *vb_ = reinterpret_cast<const bf16_t *>(a.v.ptr) + b * a.v.sb + hk * a.v.sh;
+  const int nt_all = (Sk + 63) / 64;
+  const int nt = any_g ? nt_all : 0;
+  const tile_summary_t *ksum = a.ksum + (int64_t)b * nt_all;
 
-  bf16x8 kreg[NU][4];
-  bf16x8 vreg[VCH];
-  int kbreg = kIntMax;
+  const bf16_t *kbase = reinterpret_cast<const bf16_t *>(a.k.ptr) + b * a.k.sb + hk * a.k.sh;
+  const bf16_t *vbase = reinterpret_cast<const bf16_t *>(a.v.ptr) + b * a.v.sb + hk * a.v.sh;
+  const buf_rsrc_t krs = make_rsrc(kbase, (uint32_t)(((int64_t)(Sk - 1) * a.k.ss + D) * 2));
+  const buf_rsrc_t vrs = make_rsrc(vbase, (uint32_t)(((int64_t)(Sk - 1) * a.v.ss + D) * 2));
+  const buf_rsrc_t idrs =
+      make_rsrc(a.kbm + (int64_t)b * nt_all * 64, (uint32_t)(nt_all * 64 * 4));
+  TileLoad<D, NT> kld, vld;
+  kld.init(tid, a.k.ss);
+  vld.init(tid, a.v.ss);
+  const uint32_t kstep = (uint32_t)(64 * a.k.ss * 2), vstep = (uint32_t)(64 * a.v.ss * 2);
 
+  // Next tile at or after t that some row of the workgroup can see, with its summary.
+  // (Summaries are read before a tile's asynchronous loads are issued: an ordinary
+  // load issued after them could only complete once they have.)
+  tile_summary_t sm_next = {0, 0, 0, 0};
   auto next_needed = [&](int t) {
-    while (t < nt && ksum[t].x > qmax_g) ++t;
-    return t;
-  };
-  auto fetch = [&](int t) {
-    const int j0 = t * BN;
-    load_units<D>(kreg, kb_, a.k.ss, j0, Sk, tid);
-#pragma unroll
-    for (int it = 0; it < VCH; ++it) {
-      const int c = tid + 256 * it;
-      const int row = c / CPR, col = c % CPR;
-      const int jc = min(j0 + row, Sk - 1);
-      const bf16x8 val = *reinterpret_cast<const bf16x8 *>(vb_ + (int64_t)jc * a.v.ss + col * 8);
-      vreg[it] = keep_if(j0 + row < Sk, val);
+    while (t < nt) {
+      sm_next = ksum[t];
+      if (sm_next.x <= qmax_g) break;
+      ++t;
     }
-    {
-      const int j = j0 + (tid & (BN - 1)), jc = min(j, Sk - 1);
-      const int id = a.k_blk[(int64_t)b * Sk + jc];
-      const int ok = a.k_valid[(int64_t)b * Sk + jc];
-      kbreg = (j < Sk && ok != 0) ? id : kIntMax;
-    }
+    sm_next = uniform_summary(sm_next);
+    return __builtin_amdgcn_readfirstlane(t);  // same in every lane; tell the compiler so
   };
-  auto stage = [&]() {
-    store_units<D, true, true>(kreg, Ks, Kt, tid);
-#pragma unroll
-    for (int it = 0; it < VCH; ++it) {
-      const int c = tid + 256 * it;
-      const int row = c / CPR, col = c % CPR;
-      *reinterpret_cast<bf16x8 *>(Vs + row * KP + col * 8) = vreg[it];
-    }
-    if (tid < BN) kb_s[tid] = kbreg;
+  auto issue = [&](int t, char *st) {
+    kld.issue(krs, st, (uint32_t)t * kstep, wave);
+    vld.issue(vrs, st + T::kBytes, (uint32_t)t * vstep, wave);
+    if (wave == 0) load_row64_dwords(idrs, st + 2 * T::kBytes, (uint32_t)t * 256, lane);
   };
+
+  TrLane<D> trl;
+  trl.init(lane);
 
   f32x16 dq[DB];
 #pragma unroll
@@ -207,69 +164,70 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(const BwdArgs a) {
     for (int x = 0; x < 16; ++x) dq[db][x] = 0.f;
   const float c = a.scale * kLog2e;
 
-  int t = next_needed(0);
-  if (PF && t < nt) fetch(t);
-  while (t < nt) {
-    if (!PF) fetch(t);
-    stage();
-    __syncthreads();
-    const tile_summary_t sm = ksum[t];
-    const int tn = next_needed(t + 1);
-    if (PF && tn < nt) fetch(tn);
-
-    if (sm.x <= qmax_w) {
-      const bool needmask = !(sm.z != 0 && sm.y <= qmin_w);
+  auto compute = [&](const char *st, const tile_summary_t sm) {
+    if (sm.x > qmax_w) return;  // wave-uniform: no row of this wave sees a key of the tile
+    const char *Kt = st, *Vt = st + T::kBytes;
+    const int *kb_s = reinterpret_cast<const int *>(st + 2 * T::kBytes);
+    const bool needmask = !(sm.z != 0 && sm.y <= qmin_w);
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb) {
-        f32x16 s, dp;
+    for (int mb = 0; mb < 2; ++mb) {
+      f32x16 s, dp;
 #pragma unroll
-        for (int x = 0; x < 16; ++x) s[x] = 0.f, dp[x] = 0.f;
-        const bf16_t *kp = Ks + (32 * mb + n) * KP + 8 * hh;
-        const bf16_t *vp = Vs + (32 * mb + n) * KP + 8 * hh;
-        constexpr int KB = DK < 8 ? DK : 8;  // operand reads issued ahead of the products
+      for (int x = 0; x < 16; ++x) s[x] = 0.f, dp[x] = 0.f;
+      constexpr int KB = 2;  // operand reads issued ahead of the products
 #pragma unroll
-        for (int k0 = 0; k0 < DK; k0 += KB) {
-          bf16x8 fa[KB], fb[KB];
+      for (int k0 = 0; k0 < DK; k0 += KB) {
+        bf16x8 fa[KB], fb[KB];
 #pragma unroll
-          for (int ks = 0; ks < KB; ++ks) {
-            fa[ks] = *reinterpret_cast<const bf16x8 *>(kp + 16 * (k0 + ks));
-            fb[ks] = *reinterpret_cast<const bf16x8 *>(vp + 16 * (k0 + ks));
-          }
-#pragma unroll
-          for (int ks = 0; ks < KB; ++ks) {
-            s = mfma32(fa[ks], qf[k0 + ks], s);
-            dp = mfma32(fb[ks], gof[k0 + ks], dp);
-          }
+        for (int ks = 0; ks < KB; ++ks) {
+          fa[ks] = row_operand<D>(Kt, 32 * mb + n, k0 + ks, hh);
+          fb[ks] = row_operand<D>(Vt, 32 * mb + n, k0 + ks, hh);
         }
-        float ds[16];
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-          i32x4 kb4 = {0, 0, 0, 0};
-          if (needmask) kb4 = *reinterpret_cast<const i32x4 *>(kb_s + 32 * mb + 8 * r4 + 4 * hh);
-#pragma unroll
-          for (int x = 0; x < 4; ++x) {
-            float p = fast_exp2(s[4 * r4 + x] * c - lse2);
-            if (needmask && kb4[x] > qb) p = 0.f;
-            ds[4 * r4 + x] = p * (dp[4 * r4 + x] - delta);
-          }
-        }
-        bf16x8 dsb[2];
-        dsb[0] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
-        dsb[1] = pack8(ds[8], ds[9], ds[10], ds[11], ds[12], ds[13], ds[14], ds[15]);
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const int d = 32 * db + n;
-#pragma unroll
-          for (int half = 0; half < 2; ++half) {
-            const bf16x8 ka =
-                *reinterpret_cast<const bf16x8 *>(Kt + tr_read_off(d, 2 * mb + half, hh));
-            dq[db] = mfma32(ka, dsb[half], dq[db]);
-          }
+        for (int ks = 0; ks < KB; ++ks) {
+          s = mfma32(fa[ks], qf[k0 + ks], s);
+          dp = mfma32(fb[ks], gof[k0 + ks], dp);
         }
       }
+      float ds[16];
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        i32x4 kb4 = {0, 0, 0, 0};
+        if (needmask) kb4 = *reinterpret_cast<const i32x4 *>(kb_s + 32 * mb + 8 * r4 + 4 * hh);
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          float p = fast_exp2(s[4 * r4 + x] * c - lse2);
+          if (needmask && kb4[x] > qb) p = 0.f;
+          ds[4 * r4 + x] = p * (dp[4 * r4 + x] - delta);
+        }
+      }
+      bf16x8 dsb[2];
+      dsb[0] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
+      dsb[1] = pack8(ds[8], ds[9], ds[10], ds[11], ds[12], ds[13], ds[14], ds[15]);
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        bf16x8 ka[DB];
+#pragma unroll
+        for (int db = 0; db < DB; ++db) ka[db] = tr_operand<D>(Kt, trl, 2 * mb + half, db);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) dq[db] = mfma32(ka[db], dsb[half], dq[db]);
+      }
     }
+  };
+
+  // Two LDS stages: while tile t is being used, tile t+1 streams into the other one.
+  int t = next_needed(0);
+  int stage = 0;
+  if (t < nt) issue(t, smem);
+  while (t < nt) {
+    const tile_summary_t sm = sm_next;
+    const int tn = next_needed(t + 1);
+    wait_async_loads();
     __syncthreads();
+    if (tn < nt) issue(tn, smem + (stage ^ 1) * STAGE);
+    compute(smem + stage * STAGE, sm);
     t = tn;
+    stage ^= 1;
   }
 
   if (rowok) {
@@ -288,39 +246,31 @@ __global__ __launch_bounds__(256) void bwd_dq_kernel(const BwdArgs a) {
 
 template <int D>
 constexpr size_t dq_smem_bytes() {
-  return (size_t)(2 * 64 * RowTile<D>::kPitch + D * 64) * 2 + 64 * 4 + 8 * 4;
+  return 2 * (2 * (size_t)Tile<D>::kBytes + 256);
 }
 
 // ---- dK / dV ---------------------------------------------------------------------
-template <int D, bool PF>
+template <int D>
 __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
-  constexpr int BQ = 64;
-  constexpr int KP = RowTile<D>::kPitch;
-  constexpr int DK = D / 16;
-  constexpr int DB = D / 32;
-  constexpr int NU = TileUnits<D>::NU;
+  using T = Tile<D>;
+  constexpr int DK = D / 16, DB = D / 32;
+  constexpr int STAGE = 2 * T::kBytes + 3 * 256;  // Q tile, dO tile, lse2, delta, q ids
 
-  extern __shared__ __align__(16) char smem_raw[];
-  bf16_t *Qs = reinterpret_cast<bf16_t *>(smem_raw);
-  bf16_t *Gs = Qs + BQ * KP;
-  bf16_t *Qt = Gs + BQ * KP;
-  bf16_t *Gt = Qt + D * BQ;
-  float *lse_s = reinterpret_cast<float *>(Gt + D * BQ);
-  float *delta_s = lse_s + BQ;
-  int *qb_s = reinterpret_cast<int *>(delta_s + BQ);
-  int *red_s = qb_s + BQ;
+  extern __shared__ __align__(1024) char smem[];
+  __shared__ int red_s[4];
 
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
 
-  const int Sk = a.Sk, Sq = a.Sq;
+  const int Sk = a.Sk, Sq = a.Sq, Sqp = a.Sq_pad;
   const int nkt = (Sk + 127) / 128;
   int bid = blockIdx.x;
-  const int kt = bid % nkt;
+  const int kt = __builtin_amdgcn_readfirstlane(bid % nkt);
   bid /= nkt;
-  const int hk = bid % a.Hkv;
-  const int b = bid / a.Hkv;
+  // (division results live in vector registers; say that they are uniform)
+  const int hk = __builtin_amdgcn_readfirstlane(bid % a.Hkv);
+  const int b = __builtin_amdgcn_readfirstlane(bid / a.Hkv);
 
   // ---- this lane's key -----------------------------------------------------
   const int j = kt * 128 + wave * 32 + n;
@@ -345,50 +295,48 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
   __syncthreads();
   const int kmin_g = min(min(red_s[0], red_s[1]), min(red_s[2], red_s[3]));
 
-  const int nqt = (Sq + BQ - 1) / BQ;
+  const int nqt = Sqp / 64;
   const tile_summary_t *qsum = a.qsum + (int64_t)b * nqt;
   const int nit = (kmin_g == kIntMax) ? 0 : a.G * nqt;
 
-  bf16x8 qreg[NU][4], greg[NU][4];
-  float lsereg = INFINITY, delreg = 0.f;
-  int qbreg = kIntMin;
+  const bf16_t *qb0 = reinterpret_cast<const bf16_t *>(a.q.ptr) + b * a.q.sb + (int64_t)hk * a.G * a.q.sh;
+  const bf16_t *gb0 =
+      reinterpret_cast<const bf16_t *>(a.d_o.ptr) + b * a.d_o.sb + (int64_t)hk * a.G * a.d_o.sh;
+  const uint32_t qbytes = (uint32_t)(((int64_t)(Sq - 1) * a.q.ss + D) * 2);
+  const uint32_t gbytes = (uint32_t)(((int64_t)(Sq - 1) * a.d_o.ss + D) * 2);
+  const int64_t stat0 = ((int64_t)b * a.H + (int64_t)hk * a.G) * Sqp;  // first row of (b, first head)
+  const buf_rsrc_t lrs = make_rsrc(a.lse2 + stat0, (uint32_t)(a.G * Sqp * 4));
+  const buf_rsrc_t drs = make_rsrc(a.delta + stat0, (uint32_t)(a.G * Sqp * 4));
+  const buf_rsrc_t irs = make_rsrc(a.qbm + (int64_t)b * Sqp, (uint32_t)(Sqp * 4));
+  TileLoad<D, 256> qld, gld;
+  qld.init(tid, a.q.ss);
+  gld.init(tid, a.d_o.ss);
+  const uint32_t qstep = (uint32_t)(64 * a.q.ss * 2), gstep = (uint32_t)(64 * a.d_o.ss * 2);
 
+  tile_summary_t sm_next = {0, 0, 0, 0};
   auto next_needed = [&](int it) {
     while (it < nit) {
-      const tile_summary_t s = qsum[it % nqt];
-      if (s.w > 0 && s.y >= kmin_g) break;
+      sm_next = qsum[it % nqt];
+      if (sm_next.w > 0 && sm_next.y >= kmin_g) break;
       ++it;
     }
-    return it;
+    sm_next = uniform_summary(sm_next);
+    return __builtin_amdgcn_readfirstlane(it);  // same in every lane; tell the compiler so
   };
-  auto fetch = [&](int it) {
+  auto issue = [&](int it, char *st) {
     const int g = it / nqt, qt = it - g * nqt;
-    const int h = hk * a.G + g;
-    const int i0 = qt * BQ;
-    const bf16_t *qb_ = reinterpret_cast<const bf16_t *>(a.q.ptr) + b * a.q.sb + h * a.q.sh;
-    const bf16_t *gb_ = reinterpret_cast<const bf16_t *>(a.d_o.ptr) + b * a.d_o.sb + h * a.d_o.sh;
-    load_units<D>(qreg, qb_, a.q.ss, i0, Sq, tid);
-    load_units<D>(greg, gb_, a.d_o.ss, i0, Sq, tid);
-    {
-      const int i = i0 + (tid & (BQ - 1)), ic = min(i, Sq - 1);
-      const int64_t stat = ((int64_t)b * a.H + h) * Sq + ic;
-      const float lv = a.lse[stat], dl = a.delta[stat];
-      const int id = a.q_blk[(int64_t)b * Sq + ic];
-      const bool ok = i < Sq && a.q_valid[(int64_t)b * Sq + ic] != 0;
-      lsereg = ok ? lv * kLog2e : INFINITY;
-      delreg = ok ? dl : 0.f;
-      qbreg = ok ? id : kIntMin;
-    }
+    const buf_rsrc_t qrs = make_rsrc(qb0 + (int64_t)g * a.q.sh, qbytes);
+    const buf_rsrc_t grs = make_rsrc(gb0 + (int64_t)g * a.d_o.sh, gbytes);
+    qld.issue(qrs, st, (uint32_t)qt * qstep, wave);
+    gld.issue(grs, st + T::kBytes, (uint32_t)qt * gstep, wave);
+    char *aux = st + 2 * T::kBytes;
+    if (wave == 0) load_row64_dwords(lrs, aux, (uint32_t)(g * Sqp + qt * 64) * 4, lane);
+    if (wave == 1) load_row64_dwords(drs, aux + 256, (uint32_t)(g * Sqp + qt * 64) * 4, lane);
+    if (wave == 2) load_row64_dwords(irs, aux + 512, (uint32_t)(qt * 64) * 4, lane);
   };
-  auto stage = [&]() {
-    store_units<D, true, true>(qreg, Qs, Qt, tid);
-    store_units<D, true, true>(greg, Gs, Gt, tid);
-    if (tid < BQ) {
-      lse_s[tid] = lsereg;
-      delta_s[tid] = delreg;
-      qb_s[tid] = qbreg;
-    }
-  };
+
+  TrLane<D> trl;
+  trl.init(lane);
 
   f32x16 dk[DB], dv[DB];
 #pragma unroll
@@ -397,75 +345,87 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
     for (int x = 0; x < 16; ++x) dk[db][x] = 0.f, dv[db][x] = 0.f;
   const float c = a.scale * kLog2e;
 
-  int it = next_needed(0);
-  if (PF && it < nit) fetch(it);
-  while (it < nit) {
-    if (!PF) fetch(it);
-    stage();
-    __syncthreads();
-    const tile_summary_t sm = qsum[it % nqt];
-    const int itn = next_needed(it + 1);
-    if (PF && itn < nit) fetch(itn);
-
-    if (sm.y >= kmin_w) {
-      const bool needmask = !(sm.z != 0 && allk_w != 0 && kmax_w <= sm.x);
+  auto compute = [&](const char *st, const tile_summary_t sm) {
+    if (sm.y < kmin_w) return;  // wave-uniform: no key of this wave is seen by the tile
+    const char *Qt = st, *Gt = st + T::kBytes;
+    const float *lse_s = reinterpret_cast<const float *>(st + 2 * T::kBytes);
+    const float *delta_s = lse_s + 64;
+    const int *qb_s = reinterpret_cast<const int *>(delta_s + 64);
+    const bool needmask = !(sm.z != 0 && allk_w != 0 && kmax_w <= sm.x);
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb) {
-        f32x16 s, dp;
+    for (int mb = 0; mb < 2; ++mb) {
+      f32x16 s, dp;
 #pragma unroll
-        for (int x = 0; x < 16; ++x) s[x] = 0.f, dp[x] = 0.f;
-        const bf16_t *qp = Qs + (32 * mb + n) * KP + 8 * hh;
-        const bf16_t *gp = Gs + (32 * mb + n) * KP + 8 * hh;
-        constexpr int KB = DK < 8 ? DK : 8;
+      for (int x = 0; x < 16; ++x) s[x] = 0.f, dp[x] = 0.f;
+      constexpr int KB = DK < 4 ? DK : 4;
 #pragma unroll
-        for (int k0 = 0; k0 < DK; k0 += KB) {
-          bf16x8 fa[KB], fb[KB];
+      for (int k0 = 0; k0 < DK; k0 += KB) {
+        bf16x8 fa[KB], fb[KB];
 #pragma unroll
-          for (int ks = 0; ks < KB; ++ks) {
-            fa[ks] = *reinterpret_cast<const bf16x8 *>(qp + 16 * (k0 + ks));
-            fb[ks] = *reinterpret_cast<const bf16x8 *>(gp + 16 * (k0 + ks));
-          }
-#pragma unroll
-          for (int ks = 0; ks < KB; ++ks) {
-            s = mfma32(fa[ks], kf[k0 + ks], s);
-            dp = mfma32(fb[ks], vf[k0 + ks], dp);
-          }
+        for (int ks = 0; ks < KB; ++ks) {
+          fa[ks] = row_operand<D>(Qt, 32 * mb + n, k0 + ks, hh);
+          fb[ks] = row_operand<D>(Gt, 32 * mb + n, k0 + ks, hh);
         }
-        float p[16], ds[16];
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-          const int q0 = 32 * mb + 8 * r4 + 4 * hh;
-          const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lse_s + q0);
-          const f32x4 del4 = *reinterpret_cast<const f32x4 *>(delta_s + q0);
-          i32x4 qb4 = {0, 0, 0, 0};
-          if (needmask) qb4 = *reinterpret_cast<const i32x4 *>(qb_s + q0);
-#pragma unroll
-          for (int x = 0; x < 4; ++x) {
-            float pv = fast_exp2(s[4 * r4 + x] * c - lse4[x]);
-            if (needmask && kb > qb4[x]) pv = 0.f;
-            p[4 * r4 + x] = pv;
-            ds[4 * r4 + x] = pv * (dp[4 * r4 + x] - del4[x]);
-          }
+        for (int ks = 0; ks < KB; ++ks) {
+          s = mfma32(fa[ks], kf[k0 + ks], s);
+          dp = mfma32(fb[ks], vf[k0 + ks], dp);
         }
-        bf16x8 pb[2], dsb[2];
-        pb[0] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
-        pb[1] = pack8(p[8], p[9], p[10], p[11], p[12], p[13], p[14], p[15]);
-        dsb[0] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
-        dsb[1] = pack8(ds[8], ds[9], ds[10], ds[11], ds[12], ds[13], ds[14], ds[15]);
+      }
+      float p[16], ds[16];
 #pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const int d = 32 * db + n;
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const int q0 = 32 * mb + 8 * r4 + 4 * hh;
+        const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lse_s + q0);
+        const f32x4 del4 = *reinterpret_cast<const f32x4 *>(delta_s + q0);
+        i32x4 qb4 = {0, 0, 0, 0};
+        if (needmask) qb4 = *reinterpret_cast<const i32x4 *>(qb_s + q0);
 #pragma unroll
-          for (int half = 0; half < 2; ++half) {
-            const int off = tr_read_off(d, 2 * mb + half, hh);
-            dv[db] = mfma32(*reinterpret_cast<const bf16x8 *>(Gt + off), pb[half], dv[db]);
-            dk[db] = mfma32(*reinterpret_cast<const bf16x8 *>(Qt + off), dsb[half], dk[db]);
+        for (int x = 0; x < 4; ++x) {
+          float pv = fast_exp2(s[4 * r4 + x] * c - lse4[x]);
+          if (needmask && kb > qb4[x]) pv = 0.f;
+          p[4 * r4 + x] = pv;
+          ds[4 * r4 + x] = pv * (dp[4 * r4 + x] - del4[x]);
+        }
+      }
+      bf16x8 pb[2], dsb[2];
+      pb[0] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
+      pb[1] = pack8(p[8], p[9], p[10], p[11], p[12], p[13], p[14], p[15]);
+      dsb[0] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
+      dsb[1] = pack8(ds[8], ds[9], ds[10], ds[11], ds[12], ds[13], ds[14], ds[15]);
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        constexpr int DBB = DB < 4 ? DB : 4;
+#pragma unroll
+        for (int d0 = 0; d0 < DB; d0 += DBB) {
+          bf16x8 ga[DBB], qa[DBB];
+#pragma unroll
+          for (int db = 0; db < DBB; ++db) {
+            ga[db] = tr_operand<D>(Gt, trl, 2 * mb + half, d0 + db);
+            qa[db] = tr_operand<D>(Qt, trl, 2 * mb + half, d0 + db);
+          }
+#pragma unroll
+          for (int db = 0; db < DBB; ++db) {
+            dv[d0 + db] = mfma32(ga[db], pb[half], dv[d0 + db]);
+            dk[d0 + db] = mfma32(qa[db], dsb[half], dk[d0 + db]);
           }
         }
       }
     }
+  };
+
+  int it = next_needed(0);
+  int stage = 0;
+  if (it < nit) issue(it, smem);
+  while (it < nit) {
+    const tile_summary_t sm = sm_next;
+    const int itn = next_needed(it + 1);
+    wait_async_loads();
     __syncthreads();
+    if (itn < nit) issue(itn, smem + (stage ^ 1) * STAGE);
+    compute(smem + stage * STAGE, sm);
     it = itn;
+    stage ^= 1;
   }
 
   if (jok) {
@@ -489,44 +449,44 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
 
 template <int D>
 constexpr size_t dkv_smem_bytes() {
-  return (size_t)(2 * 64 * RowTile<D>::kPitch + 2 * D * 64) * 2 + 3 * 64 * 4 + 8 * 4;
+  return 2 * (2 * (size_t)Tile<D>::kBytes + 3 * 256);
 }
 
-template <int D, bool PF>
+template <int D, int NWQ>
 static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
-  {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(&bwd_dq_kernel<D, PF>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)dq_smem_bytes<D>()) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void *>(&bwd_dkv_kernel<D, PF>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                            (int)dkv_smem_bytes<D>()) != hipSuccess)
-      return BCATTN_ERR_LAUNCH;
+  if (hipFuncSetAttribute(reinterpret_cast<const void *>(&bwd_dq_kernel<D, NWQ>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)dq_smem_bytes<D>()) != hipSuccess ||
+      hipFuncSetAttribute(reinterpret_cast<const void *>(&bwd_dkv_kernel<D>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)dkv_smem_bytes<D>()) != hipSuccess)
+    return BCATTN_ERR_LAUNCH;
+  if (a.stages & BCATTN_BWD_DELTA) {
+    constexpr int RPB = 256 / (D / 8);
+    const int64_t rows = (int64_t)a.B * a.H * a.Sq_pad;
+    hipLaunchKernelGGL(bwd_prep_kernel<D>, dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, a);
   }
-  constexpr int RPB = 256 / (D / 8);
-  const int64_t rows = (int64_t)a.B * a.Sq * a.H;
-  if (a.stages & BCATTN_BWD_DELTA)
-    hipLaunchKernelGGL(bwd_delta_kernel<D>, dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, a);
-  const int R = a.G * a.Sq;
-  const int ntile_r = (R + 127) / 128;
-  if (a.stages & BCATTN_BWD_DQ)
-    hipLaunchKernelGGL((bwd_dq_kernel<D, PF>), dim3((unsigned)(ntile_r * a.Hkv * a.B)), dim3(256),
-                     dq_smem_bytes<D>(), st, a);
-  const int nkt = (a.Sk + 127) / 128;
-  if (a.stages & BCATTN_BWD_DKV)
-    hipLaunchKernelGGL((bwd_dkv_kernel<D, PF>), dim3((unsigned)(nkt * a.Hkv * a.B)), dim3(256),
-                     dkv_smem_bytes<D>(), st, a);
+  if (a.stages & BCATTN_BWD_DQ) {
+    const int R = a.G * a.Sq;
+    const int ntile_r = (R + 32 * NWQ - 1) / (32 * NWQ);
+    hipLaunchKernelGGL((bwd_dq_kernel<D, NWQ>), dim3((unsigned)(ntile_r * a.Hkv * a.B)), dim3(64 * NWQ),
+                       dq_smem_bytes<D>(), st, a);
+  }
+  if (a.stages & BCATTN_BWD_DKV) {
+    const int nkt = (a.Sk + 127) / 128;
+    hipLaunchKernelGGL((bwd_dkv_kernel<D>), dim3((unsigned)(nkt * a.Hkv * a.B)), dim3(256),
+                       dkv_smem_bytes<D>(), st, a);
+  }
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
 }
 
 int launch_bwd_bf16(const BwdArgs &a, int D, hipStream_t st) {
+  const int R = a.G * a.Sq;
   switch (D) {
     case 64:
-      return launch_bwd_d<64, true>(a, st);
+      return launch_bwd_d<64, 4>(a, st);
     case 128:
-      return launch_bwd_d<128, true>(a, st);
+      return R >= 1024 ? launch_bwd_d<128, 8>(a, st) : launch_bwd_d<128, 4>(a, st);
     case 256:
-      return launch_bwd_d<256, false>(a, st);
+      return launch_bwd_d<256, 4>(a, st);
     default:
       return BCATTN_ERR_UNSUPPORTED;
   }

@@ -32,6 +32,17 @@ constexpr int kSumTile = 64;
 // the tile is in range and valid, w = number of valid keys.
 typedef i32x4 tile_summary_t;
 
+// A summary read through a uniform address is the same in every lane; moving it
+// to scalar registers makes the branches on it scalar branches.
+__device__ __forceinline__ tile_summary_t uniform_summary(tile_summary_t s) {
+  tile_summary_t r;
+  r.x = __builtin_amdgcn_readfirstlane(s.x);
+  r.y = __builtin_amdgcn_readfirstlane(s.y);
+  r.z = __builtin_amdgcn_readfirstlane(s.z);
+  r.w = __builtin_amdgcn_readfirstlane(s.w);
+  return r;
+}
+
 // D(32x32 fp32) += A(32x16 bf16) * B(16x32 bf16).
 // Lane l supplies A[row l%32][k 8*(l/32)..+7] and B[k 8*(l/32)..+7][col l%32];
 // it receives D[row 8*(r/4) + 4*(l/32) + r%4][col l%32] in register r.
@@ -167,7 +178,8 @@ struct FwdArgs {
   float *lse;
   const int32_t *q_blk, *k_blk;
   const uint8_t *q_valid, *k_valid;
-  const tile_summary_t *ksum;  // (B, ceil(Sk/64))
+  const tile_summary_t *ksum;  // (B, nt): key tiles, segment 0 first, never straddling
+  const int32_t *kbm;          // (B, nt, 64): block id per tile slot, INT_MAX where invalid / padding
   int B, Sq, Sk0, Sk, H, Hkv, G;
   float scale;
 };
@@ -177,19 +189,24 @@ struct BwdArgs {
   void *dq, *dk, *dv;
   int64_t dq_sb, dq_ss, dq_sh, dk_sb, dk_ss, dk_sh, dv_sb, dv_ss, dv_sh;
   const float *lse;
-  float *delta;  // (B,H,Sq)
+  float *delta;  // (B,H,Sq_pad): row sums of O*dO, 0 on rows that take no part
+  float *lse2;   // (B,H,Sq_pad): log2e*LSE, +inf on rows that take no part
   const int32_t *q_blk, *k_blk;
   const uint8_t *q_valid, *k_valid;
   const tile_summary_t *ksum;  // (B, ceil(Sk/64))
   const tile_summary_t *qsum;  // (B, ceil(Sq/64))
+  const int32_t *kbm;          // (B, ceil(Sk/64), 64): key ids, INT_MAX where invalid / padding
+  const int32_t *qbm;          // (B, Sq_pad): query ids, INT_MIN where invalid / padding
   int B, Sq, Sk, H, Hkv, G;
+  int Sq_pad;  // Sq rounded up to whole 64-row tiles
   float scale;
   int stages;  // bit set of bcattn_bwd_stage, never 0 here
 };
 
 // kernel launchers, one translation unit each
-int launch_summary(const int32_t *blk, const uint8_t *valid, int B, int S, tile_summary_t *out,
-                   hipStream_t st);
+// Tile summaries and merged ids of a sequence given as two segments (n0 rows, then S - n0).
+int launch_summary(const int32_t *blk, const uint8_t *valid, int B, int n0, int S, int fill,
+                   tile_summary_t *sum, int32_t *merged, hipStream_t st);
 int launch_fwd_bf16(const FwdArgs &a, int D, hipStream_t st);
 int launch_fwd_f32(const FwdArgs &a, int D, hipStream_t st);
 int launch_bwd_bf16(const BwdArgs &a, int D, hipStream_t st);
@@ -202,6 +219,6 @@ struct SplitArgs {
   int tiles_per_split;  // 64-key tiles per split
 };
 int launch_fwd_kvcache_bf16(const FwdArgs &a, const SplitArgs &s, int D, hipStream_t st);
-size_t kvcache_workspace_bytes(int B, int Sq, int Sk, int H, int Hkv, int D, int *nsplit_out);
+size_t kvcache_workspace_bytes(int B, int Sq, int Sk0, int Sk, int H, int Hkv, int D, int *nsplit_out);
 
 }  // namespace bcattn

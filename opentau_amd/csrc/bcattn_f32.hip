@@ -42,24 +42,6 @@ __device__ __forceinline__ void load_rows_f32(float *dst, int pitch, const float
   }
 }
 
-// Same for keys that come in two segments.
-__device__ __forceinline__ void load_rows2_f32(float *dst, int pitch, const float *b0, int64_t s0,
-                                               const float *b1, int64_t s1, int n0, int row0, int nrows,
-                                               int limit, int D, int tid) {
-  const int n4 = D / 4;
-  for (int idx = tid; idx < nrows * n4; idx += 256) {
-    const int row = idx / n4, c4 = idx - row * n4;
-    const int j = row0 + row;
-    f32x4 v = {0.f, 0.f, 0.f, 0.f};
-    if (j < limit) {
-      const float *p = j < n0 ? b0 + (int64_t)j * s0 : b1 + (int64_t)(j - n0) * s1;
-      v = *reinterpret_cast<const f32x4 *>(p + 4 * c4);
-    }
-    float *d = dst + row * pitch + 4 * c4;
-    d[0] = v[0], d[1] = v[1], d[2] = v[2], d[3] = v[3];
-  }
-}
-
 __global__ __launch_bounds__(256) void fwd_f32_kernel(const FwdArgs a, const int D) {
   extern __shared__ __align__(16) float smf[];
   const int KP = D + 1;
@@ -93,7 +75,9 @@ __global__ __launch_bounds__(256) void fwd_f32_kernel(const FwdArgs a, const int
   const float *v0b = reinterpret_cast<const float *>(a.v0.ptr) + b * a.v0.sb + hk * a.v0.sh;
   const float *k1b = reinterpret_cast<const float *>(a.k1.ptr) + b * a.k1.sb + hk * a.k1.sh;
   const float *v1b = reinterpret_cast<const float *>(a.v1.ptr) + b * a.v1.sb + hk * a.v1.sh;
-  const tile_summary_t *ksum = a.ksum + (int64_t)b * ((Sk + kSumTile - 1) / kSumTile);
+  const int nt0s = (a.Sk0 + kSumTile - 1) / kSumTile;  // summary tiles of segment 0
+  const tile_summary_t *ksum =
+      a.ksum + (int64_t)b * (nt0s + (Sk - a.Sk0 + kSumTile - 1) / kSumTile);
 
   float oacc[F_MAXX];
 #pragma unroll
@@ -101,46 +85,52 @@ __global__ __launch_bounds__(256) void fwd_f32_kernel(const FwdArgs a, const int
   float m = -INFINITY, l = 0.f;
   const float c = a.scale * kLog2e;
 
-  const int nt = (Sk + F_BC - 1) / F_BC;
-  for (int t = 0; t < nt; ++t) {
-    if (ksum[(t * F_BC) / kSumTile].x > qmax_g) continue;  // uniform over the workgroup
-    const int j0 = t * F_BC;
-    __syncthreads();
-    load_rows2_f32(Ks, KP, k0b, a.k0.ss, k1b, a.k1.ss, a.Sk0, j0, F_BC, Sk, D, tid);
-    load_rows2_f32(Vs, D, v0b, a.v0.ss, v1b, a.v1.ss, a.Sk0, j0, F_BC, Sk, D, tid);
-    if (tid < F_BC) {
-      const int j = j0 + tid;
-      kb_s[tid] = (j < Sk && a.k_valid[(int64_t)b * Sk + j]) ? a.k_blk[(int64_t)b * Sk + j] : kIntMax;
-    }
-    __syncthreads();
-    float s0 = 0.f, s1 = 0.f;
-    const float *qr = Qs + ri * D, *kr0 = Ks + cg * KP, *kr1 = Ks + (cg + 16) * KP;
-    for (int d = 0; d < D; ++d) {
-      const float qd = qr[d];
-      s0 = fmaf(qd, kr0[d], s0);
-      s1 = fmaf(qd, kr1[d], s1);
-    }
-    if (!qv || kb_s[cg] > qb) s0 = -INFINITY;
-    if (!qv || kb_s[cg + 16] > qb) s1 = -INFINITY;
-    const float mloc = grp16_max(fmaxf(s0, s1));
-    const float mnew = fmaxf(m, mloc);
-    const float moff = (mnew == -INFINITY) ? 0.f : mnew * c;
-    const float corr = fast_exp2(m * c - moff);
-    const float p0 = fast_exp2(s0 * c - moff), p1 = fast_exp2(s1 * c - moff);
-    l = l * corr + grp16_sum(p0 + p1);
-    m = mnew;
-    Ps[ri * F_BC + cg] = p0;
-    Ps[ri * F_BC + cg + 16] = p1;
-    __syncthreads();
-#pragma unroll
-    for (int x = 0; x < F_MAXX; ++x)
-      if (x < nx) {
-        float acc = oacc[x] * corr;
-        const float *vcol = Vs + cg + 16 * x;
-        const float *pr = Ps + ri * F_BC;
-        for (int j = 0; j < F_BC; ++j) acc = fmaf(pr[j], vcol[j * D], acc);
-        oacc[x] = acc;
+  // The two key segments are walked one after the other; tiles do not straddle them.
+  for (int seg = 0; seg < 2; ++seg) {
+    const int len = seg ? Sk - a.Sk0 : a.Sk0;
+    const int base = seg ? a.Sk0 : 0;
+    const float *kseg = seg ? k1b : k0b, *vseg = seg ? v1b : v0b;
+    const int64_t kss = seg ? a.k1.ss : a.k0.ss, vss = seg ? a.v1.ss : a.v0.ss;
+    for (int j0 = 0; j0 < len; j0 += F_BC) {
+      if (ksum[(seg ? nt0s : 0) + j0 / kSumTile].x > qmax_g) continue;  // uniform over the workgroup
+      __syncthreads();
+      load_rows_f32(Ks, KP, kseg, kss, j0, F_BC, len, D, tid);
+      load_rows_f32(Vs, D, vseg, vss, j0, F_BC, len, D, tid);
+      if (tid < F_BC) {
+        const int j = j0 + tid;
+        kb_s[tid] = (j < len && a.k_valid[(int64_t)b * Sk + base + j]) ? a.k_blk[(int64_t)b * Sk + base + j]
+                                                                       : kIntMax;
       }
+      __syncthreads();
+      float s0 = 0.f, s1 = 0.f;
+      const float *qr = Qs + ri * D, *kr0 = Ks + cg * KP, *kr1 = Ks + (cg + 16) * KP;
+      for (int d = 0; d < D; ++d) {
+        const float qd = qr[d];
+        s0 = fmaf(qd, kr0[d], s0);
+        s1 = fmaf(qd, kr1[d], s1);
+      }
+      if (!qv || kb_s[cg] > qb) s0 = -INFINITY;
+      if (!qv || kb_s[cg + 16] > qb) s1 = -INFINITY;
+      const float mloc = grp16_max(fmaxf(s0, s1));
+      const float mnew = fmaxf(m, mloc);
+      const float moff = (mnew == -INFINITY) ? 0.f : mnew * c;
+      const float corr = fast_exp2(m * c - moff);
+      const float p0 = fast_exp2(s0 * c - moff), p1 = fast_exp2(s1 * c - moff);
+      l = l * corr + grp16_sum(p0 + p1);
+      m = mnew;
+      Ps[ri * F_BC + cg] = p0;
+      Ps[ri * F_BC + cg + 16] = p1;
+      __syncthreads();
+#pragma unroll
+      for (int x = 0; x < F_MAXX; ++x)
+        if (x < nx) {
+          float acc = oacc[x] * corr;
+          const float *vcol = Vs + cg + 16 * x;
+          const float *pr = Ps + ri * F_BC;
+          for (int j = 0; j < F_BC; ++j) acc = fmaf(pr[j], vcol[j * D], acc);
+          oacc[x] = acc;
+        }
+    }
   }
 
   if (rowok) {

@@ -10,7 +10,7 @@
 // softmax reduction over keys is in-lane plus one exchange with lane^32, and so
 // that the 32x32 accumulator of S^T is already laid out as the B operand of
 // O^T = V^T P^T.  K tiles sit in LDS as rows, V tiles transposed.
-#include "bcattn_common.h"
+#include "bcattn_tiles.h"
 
 namespace bcattn {
 
@@ -21,36 +21,30 @@ namespace bcattn {
 // (batch, kv head) problems with few query rows fill the chip.
 template <int D, int NW, bool SPLIT>
 __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, const SplitArgs sp) {
-  constexpr int BN = 64;
+  using T = Tile<D>;
   constexpr int NT = 64 * NW;   // threads
   constexpr int BM = 32 * NW;   // packed query rows per workgroup
-  constexpr int KP = RowTile<D>::kPitch;
-  constexpr int DK = D / 16;   // contraction steps of K Q^T
-  constexpr int DB = D / 32;   // 32-row blocks of O^T
-  constexpr int CPR = D / 8;   // 16-byte chunks per row
-  constexpr int KCH = (BN * CPR) / NT;
-  constexpr int VUNITS = 16 * CPR;  // 4x8 transposition units per V tile
-  constexpr int VUN = (VUNITS + NT - 1) / NT;
-  static_assert((BN * CPR) % NT == 0, "K tile must divide over the threads");
+  constexpr int DK = D / 16;    // contraction steps of K Q^T
+  constexpr int DB = D / 32;    // 32-row blocks of O^T
+  constexpr int STAGE = 2 * T::kBytes + 256;  // K tile, V tile, 64 key ids
 
-  __shared__ __align__(16) bf16_t Ks[BN * KP];
-  __shared__ __align__(16) bf16_t Vt[D * BN];
-  __shared__ __align__(16) int kb_s[BN];
+  extern __shared__ __align__(1024) char smem[];
   __shared__ int red_s[2 * NW];
 
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
 
   const int R = a.G * a.Sq;
   const int ntile_r = (R + BM - 1) / BM;
   int bid = blockIdx.x;
-  const int tile = bid % ntile_r;
+  const int tile = __builtin_amdgcn_readfirstlane(bid % ntile_r);
   bid /= ntile_r;
-  const int split = SPLIT ? bid % sp.nsplit : 0;
+  const int split = SPLIT ? __builtin_amdgcn_readfirstlane(bid % sp.nsplit) : 0;
   if (SPLIT) bid /= sp.nsplit;
-  const int hk = bid % a.Hkv;
-  const int b = bid / a.Hkv;
+  // (division results live in vector registers; say that they are uniform)
+  const int hk = __builtin_amdgcn_readfirstlane(bid % a.Hkv);
+  const int b = __builtin_amdgcn_readfirstlane(bid / a.Hkv);
 
   // ---- this lane's query row ------------------------------------------------
   const int r = tile * BM + wave * 32 + n;
@@ -85,8 +79,10 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
     any_g |= red_s[NW + x];
   }
 
-  const int Sk = a.Sk;
-  const int nt_all = (Sk + BN - 1) / BN;
+  // Key tiles never straddle the two key segments: tiles [0, nt0) cover segment 0,
+  // tiles [nt0, nt0+nt1) segment 1, each padded (zero rows, invalid ids) at its end.
+  const int nt0 = (a.Sk0 + 63) / 64;
+  const int nt_all = nt0 + (a.Sk - a.Sk0 + 63) / 64;
   const int t_first = SPLIT ? split * sp.tiles_per_split : 0;
   const int nt = !any_g ? 0 : (SPLIT ? min(nt_all, t_first + sp.tiles_per_split) : nt_all);
   const tile_summary_t *ksum = a.ksum + (int64_t)b * nt_all;
@@ -95,66 +91,45 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   const bf16_t *v0b = reinterpret_cast<const bf16_t *>(a.v0.ptr) + b * a.v0.sb + hk * a.v0.sh;
   const bf16_t *k1b = reinterpret_cast<const bf16_t *>(a.k1.ptr) + b * a.k1.sb + hk * a.k1.sh;
   const bf16_t *v1b = reinterpret_cast<const bf16_t *>(a.v1.ptr) + b * a.v1.sb + hk * a.v1.sh;
-  const int Sk0 = a.Sk0;
-  const int32_t *kblk_b = a.k_blk + (int64_t)b * Sk;
-  const uint8_t *kval_b = a.k_valid + (int64_t)b * Sk;
+  const int n0 = a.Sk0 > 0 ? a.Sk0 : 1, n1 = a.Sk - a.Sk0 > 0 ? a.Sk - a.Sk0 : 1;
+  const buf_rsrc_t k0rs = make_rsrc(k0b, (uint32_t)(((int64_t)(n0 - 1) * a.k0.ss + D) * 2));
+  const buf_rsrc_t v0rs = make_rsrc(v0b, (uint32_t)(((int64_t)(n0 - 1) * a.v0.ss + D) * 2));
+  const buf_rsrc_t k1rs = make_rsrc(k1b, (uint32_t)(((int64_t)(n1 - 1) * a.k1.ss + D) * 2));
+  const buf_rsrc_t v1rs = make_rsrc(v1b, (uint32_t)(((int64_t)(n1 - 1) * a.v1.ss + D) * 2));
+  const buf_rsrc_t idrs =
+      make_rsrc(a.kbm + (int64_t)b * nt_all * 64, (uint32_t)(nt_all * 64 * 4));
+  TileLoad<D, NT> k0ld, v0ld, k1ld, v1ld;
+  k0ld.init(tid, a.k0.ss);
+  v0ld.init(tid, a.v0.ss);
+  k1ld.init(tid, a.k1.ss);
+  v1ld.init(tid, a.v1.ss);
 
-  bf16x8 kreg[KCH];
-  bf16x8 vreg[VUN][4];
-  int kbreg = kIntMax;
-
+  // Next tile at or after t that some row of the workgroup can see, with its summary.
+  // (Summaries are read before a tile's asynchronous loads are issued: an ordinary
+  // load issued after them could only complete once they have.)
+  tile_summary_t sm_next = {0, 0, 0, 0};
   auto next_needed = [&](int t) {
-    while (t < nt && ksum[t].x > qmax_g) ++t;
-    return t;
+    while (t < nt) {
+      sm_next = ksum[t];
+      if (sm_next.x <= qmax_g) break;
+      ++t;
+    }
+    sm_next = uniform_summary(sm_next);
+    return __builtin_amdgcn_readfirstlane(t);  // same in every lane; tell the compiler so
+  };
+  auto issue = [&](int t, char *st) {
+    if (t < nt0) {
+      k0ld.issue(k0rs, st, (uint32_t)(t * 64 * a.k0.ss * 2), wave);
+      v0ld.issue(v0rs, st + T::kBytes, (uint32_t)(t * 64 * a.v0.ss * 2), wave);
+    } else {
+      k1ld.issue(k1rs, st, (uint32_t)((t - nt0) * 64 * a.k1.ss * 2), wave);
+      v1ld.issue(v1rs, st + T::kBytes, (uint32_t)((t - nt0) * 64 * a.v1.ss * 2), wave);
+    }
+    if (wave == 0) load_row64_dwords(idrs, st + 2 * T::kBytes, (uint32_t)t * 256, lane);
   };
 
-  // Global loads of one tile into registers (consumed by stage() one iteration later).
-  auto prefetch = [&](int t) {
-    const int j0 = t * BN;
-#pragma unroll
-    for (int it = 0; it < KCH; ++it) {
-      const int c = tid + NT * it;
-      const int row = c / CPR, col = c % CPR;
-      const int j = j0 + row, jc = min(j, Sk - 1);
-      const bf16x8 val =
-          *reinterpret_cast<const bf16x8 *>(seg_row(k0b, a.k0.ss, k1b, a.k1.ss, Sk0, jc) + col * 8);
-      kreg[it] = keep_if(j < Sk, val);
-    }
-#pragma unroll
-    for (int it = 0; it < VUN; ++it) {
-      const int u = min(tid + NT * it, VUNITS - 1);
-      const int dch = u % CPR, kg = u / CPR;
-#pragma unroll
-      for (int x = 0; x < 4; ++x) {
-        const int j = j0 + 4 * kg + x, jc = min(j, Sk - 1);
-        const bf16x8 val =
-            *reinterpret_cast<const bf16x8 *>(seg_row(v0b, a.v0.ss, v1b, a.v1.ss, Sk0, jc) + dch * 8);
-        vreg[it][x] = keep_if(j < Sk, val);
-      }
-    }
-    {
-      const int j = j0 + (tid & (BN - 1)), jc = min(j, Sk - 1);
-      const int id = kblk_b[jc];
-      const int ok = kval_b[jc];
-      kbreg = (j < Sk && ok != 0) ? id : kIntMax;
-    }
-  };
-
-  auto stage = [&]() {
-#pragma unroll
-    for (int it = 0; it < KCH; ++it) {
-      const int c = tid + NT * it;
-      const int row = c / CPR, col = c % CPR;
-      *reinterpret_cast<bf16x8 *>(Ks + row * KP + col * 8) = kreg[it];
-    }
-#pragma unroll
-    for (int it = 0; it < VUN; ++it) {
-      const int u = tid + NT * it;
-      const int dch = u % CPR, kg = u / CPR;
-      if (u < VUNITS) tr_store_4x8(Vt, 8 * dch, kg, vreg[it][0], vreg[it][1], vreg[it][2], vreg[it][3]);
-    }
-    if (tid < BN) kb_s[tid] = kbreg;
-  };
+  TrLane<D> trl;
+  trl.init(lane);
 
   // ---- running state ---------------------------------------------------------
   f32x16 o[DB];
@@ -166,82 +141,103 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   float l = 0.f;        // this lane half's share of the running sum
   const float c = a.scale * kLog2e;
 
-  int t = next_needed(t_first);
-  if (t < nt) prefetch(t);
-  while (t < nt) {
-    stage();
-    __syncthreads();
-    const tile_summary_t sm = ksum[t];
-    const int tn = next_needed(t + 1);
-    if (tn < nt) prefetch(tn);
-
-    if (sm.x <= qmax_w) {  // wave-uniform: some row of this wave sees some key of the tile
-      f32x16 s[2];
+  auto compute = [&](const char *st, const tile_summary_t sm) {
+    if (sm.x > qmax_w) return;  // wave-uniform: no row of this wave sees a key of the tile
+    const char *Kt = st, *Vt = st + T::kBytes;
+    const int *kb_s = reinterpret_cast<const int *>(st + 2 * T::kBytes);
+    // Two independent accumulator chains (the two 32-key halves) are interleaved:
+    // back-to-back products on one accumulator would each wait for the previous one.
+    f32x16 s[2];
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb) {
+    for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-        for (int x = 0; x < 16; ++x) s[mb][x] = 0.f;
-        const bf16_t *kp = Ks + (32 * mb + n) * KP + 8 * hh;
-        bf16x8 ka[DK];
+      for (int x = 0; x < 16; ++x) s[mb][x] = 0.f;
+    {
+      constexpr int KB = DK < 4 ? DK : 4;
 #pragma unroll
-        for (int ks = 0; ks < DK; ++ks) ka[ks] = *reinterpret_cast<const bf16x8 *>(kp + 16 * ks);
+      for (int k0 = 0; k0 < DK; k0 += KB) {
+        bf16x8 ka0[KB], ka1[KB];
 #pragma unroll
-        for (int ks = 0; ks < DK; ++ks) s[mb] = mfma32(ka[ks], qf[ks], s[mb]);
+        for (int ks = 0; ks < KB; ++ks) {
+          ka0[ks] = row_operand<D>(Kt, n, k0 + ks, hh);
+          ka1[ks] = row_operand<D>(Kt, 32 + n, k0 + ks, hh);
+        }
+#pragma unroll
+        for (int ks = 0; ks < KB; ++ks) {
+          s[0] = mfma32(ka0[ks], qf[k0 + ks], s[0]);
+          s[1] = mfma32(ka1[ks], qf[k0 + ks], s[1]);
+        }
       }
-      const bool needmask = !(sm.z != 0 && sm.y <= qmin_w);
-      if (needmask) {
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-          for (int r4 = 0; r4 < 4; ++r4) {
-            const i32x4 kb4 = *reinterpret_cast<const i32x4 *>(kb_s + 32 * mb + 8 * r4 + 4 * hh);
-#pragma unroll
-            for (int x = 0; x < 4; ++x)
-              if (kb4[x] > qb) s[mb][4 * r4 + x] = -INFINITY;
-          }
-      }
-      float mloc = s[0][0];
+    }
+    const bool needmask = !(sm.z != 0 && sm.y <= qmin_w);
+    if (needmask) {
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb)
 #pragma unroll
-        for (int x = 0; x < 16; ++x) mloc = fmaxf(mloc, s[mb][x]);
-      mloc = fmaxf(mloc, swap32(mloc));
-      const float mnew = fmaxf(m, mloc);
-      const float moff = (mnew == -INFINITY) ? 0.f : mnew * c;
-      if (__any(mnew > m)) {
-        const float corr = fast_exp2(m * c - moff);
-        l *= corr;
+        for (int r4 = 0; r4 < 4; ++r4) {
+          const i32x4 kb4 = *reinterpret_cast<const i32x4 *>(kb_s + 32 * mb + 8 * r4 + 4 * hh);
 #pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-          for (int x = 0; x < 16; ++x) o[db][x] *= corr;
-      }
-      m = mnew;
-      bf16x8 pb[4];
-#pragma unroll
-      for (int mb = 0; mb < 2; ++mb) {
-        float p[16];
-#pragma unroll
-        for (int x = 0; x < 16; ++x) {
-          p[x] = fast_exp2(s[mb][x] * c - moff);
-          l += p[x];
+          for (int x = 0; x < 4; ++x)
+            if (kb4[x] > qb) s[mb][4 * r4 + x] = -INFINITY;
         }
-        pb[2 * mb] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
-        pb[2 * mb + 1] = pack8(p[8], p[9], p[10], p[11], p[12], p[13], p[14], p[15]);
+    }
+    float mloc = s[0][0];
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int x = 0; x < 16; ++x) mloc = fmaxf(mloc, s[mb][x]);
+    mloc = fmaxf(mloc, swap32(mloc));
+    const float mnew = fmaxf(m, mloc);
+    const float moff = (mnew == -INFINITY) ? 0.f : mnew * c;
+    if (__any(mnew > m)) {
+      const float corr = fast_exp2(m * c - moff);
+      l *= corr;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int x = 0; x < 16; ++x) o[db][x] *= corr;
+    }
+    m = mnew;
+    bf16x8 pb[4];
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) {
+      float p[16];
+#pragma unroll
+      for (int x = 0; x < 16; ++x) {
+        p[x] = fast_exp2(s[mb][x] * c - moff);
+        l += p[x];
       }
+      pb[2 * mb] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
+      pb[2 * mb + 1] = pack8(p[8], p[9], p[10], p[11], p[12], p[13], p[14], p[15]);
+    }
+    // O^T += V^T P^T: the DB accumulators are independent, so the key steps run outermost.
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const int d = 32 * db + n;
-        bf16x8 va[4];
+    for (int kk = 0; kk < 4; ++kk) {
+      constexpr int DBB = DB < 4 ? DB : 4;
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk)
-          va[kk] = *reinterpret_cast<const bf16x8 *>(Vt + tr_read_off(d, kk, hh));
+      for (int d0 = 0; d0 < DB; d0 += DBB) {
+        bf16x8 va[DBB];
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) o[db] = mfma32(va[kk], pb[kk], o[db]);
+        for (int db = 0; db < DBB; ++db) va[db] = tr_operand<D>(Vt, trl, kk, d0 + db);
+#pragma unroll
+        for (int db = 0; db < DBB; ++db) o[d0 + db] = mfma32(va[db], pb[kk], o[d0 + db]);
       }
     }
+  };
+
+  // Two LDS stages: while tile t is being used, tile t+1 streams into the other one.
+  int t = next_needed(t_first);
+  int stage = 0;
+  if (t < nt) issue(t, smem);
+  while (t < nt) {
+    const tile_summary_t sm = sm_next;
+    const int tn = next_needed(t + 1);
+    wait_async_loads();
     __syncthreads();
+    if (tn < nt) issue(tn, smem + (stage ^ 1) * STAGE);
+    compute(smem + stage * STAGE, sm);
     t = tn;
+    stage ^= 1;
   }
 
   // ---- epilogue ----------------------------------------------------------------
@@ -284,6 +280,11 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
         *reinterpret_cast<bf16x4 *>(optr + 32 * db + 8 * r4 + 4 * hh) = w;
       }
   }
+}
+
+template <int D>
+constexpr size_t fwd_smem_bytes() {
+  return 2 * (2 * (size_t)Tile<D>::kBytes + 256);
 }
 
 // Merge the per-split partials: one thread per (packed row, 4 head_dim columns).
@@ -329,34 +330,39 @@ __global__ __launch_bounds__(256) void fwd_combine_kernel(const FwdArgs a, const
     a.lse[((int64_t)b * a.H + h) * a.Sq + i] = has ? mx * a.scale + __logf(lsum) : 0.f;
 }
 
-int launch_fwd_bf16(const FwdArgs &a, int D, hipStream_t st) {
+template <int D, int NW, bool SPLIT>
+static int launch_fwd_t(const FwdArgs &a, const SplitArgs &sp, hipStream_t st) {
+  if (hipFuncSetAttribute(reinterpret_cast<const void *>(&fwd_bf16_kernel<D, NW, SPLIT>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)fwd_smem_bytes<D>()) != hipSuccess)
+    return BCATTN_ERR_LAUNCH;
   const int R = a.G * a.Sq;
-  const SplitArgs sp{nullptr, nullptr, 1, 0};
-  auto grid = [&](int bm) { return dim3((unsigned)(((R + bm - 1) / bm) * a.Hkv * a.B)); };
-  switch (D) {
-    case 64:
-      hipLaunchKernelGGL((fwd_bf16_kernel<64, 4, false>), grid(128), dim3(256), 0, st, a, sp);
-      break;
-    case 128:
-      if (R >= 1024)
-        hipLaunchKernelGGL((fwd_bf16_kernel<128, 8, false>), grid(256), dim3(512), 0, st, a, sp);
-      else
-        hipLaunchKernelGGL((fwd_bf16_kernel<128, 4, false>), grid(128), dim3(256), 0, st, a, sp);
-      break;
-    case 256:
-      hipLaunchKernelGGL((fwd_bf16_kernel<256, 4, false>), grid(128), dim3(256), 0, st, a, sp);
-      break;
-    default:
-      return BCATTN_ERR_UNSUPPORTED;
-  }
+  const int ntile_r = (R + 32 * NW - 1) / (32 * NW);
+  hipLaunchKernelGGL((fwd_bf16_kernel<D, NW, SPLIT>),
+                     dim3((unsigned)(ntile_r * (SPLIT ? sp.nsplit : 1) * a.Hkv * a.B)), dim3(64 * NW),
+                     fwd_smem_bytes<D>(), st, a, sp);
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
 }
 
+int launch_fwd_bf16(const FwdArgs &a, int D, hipStream_t st) {
+  const int R = a.G * a.Sq;
+  const SplitArgs sp{nullptr, nullptr, 1, 0};
+  switch (D) {
+    case 64:
+      return launch_fwd_t<64, 4, false>(a, sp, st);
+    case 128:
+      return R >= 1024 ? launch_fwd_t<128, 8, false>(a, sp, st) : launch_fwd_t<128, 4, false>(a, sp, st);
+    case 256:
+      return launch_fwd_t<256, 4, false>(a, sp, st);
+    default:
+      return BCATTN_ERR_UNSUPPORTED;
+  }
+}
+
 // How many ways to split the key axis so that about 1.5 workgroups per CU exist.
-static void plan_split(int B, int Sq, int Sk, int H, int Hkv, int *nsplit, int *tps) {
+static void plan_split(int B, int Sq, int Sk0, int Sk, int H, int Hkv, int *nsplit, int *tps) {
   const int R = (H / Hkv) * Sq;
   const int base = B * Hkv * ((R + 127) / 128);
-  const int ntiles = (Sk + 63) / 64;
+  const int ntiles = (Sk0 + 63) / 64 + (Sk - Sk0 + 63) / 64;
   int want = (384 + base - 1) / base;
   if (want < 1) want = 1;
   if (want > ntiles) want = ntiles;
@@ -364,9 +370,9 @@ static void plan_split(int B, int Sq, int Sk, int H, int Hkv, int *nsplit, int *
   *nsplit = (ntiles + *tps - 1) / *tps;
 }
 
-size_t kvcache_workspace_bytes(int B, int Sq, int Sk, int H, int Hkv, int D, int *nsplit_out) {
+size_t kvcache_workspace_bytes(int B, int Sq, int Sk0, int Sk, int H, int Hkv, int D, int *nsplit_out) {
   int ns, tps;
-  plan_split(B, Sq, Sk, H, Hkv, &ns, &tps);
+  plan_split(B, Sq, Sk0, Sk, H, Hkv, &ns, &tps);
   *nsplit_out = ns;
   if (ns <= 1) return 0;
   const size_t R = (size_t)(H / Hkv) * Sq;
@@ -377,9 +383,8 @@ size_t kvcache_workspace_bytes(int B, int Sq, int Sk, int H, int Hkv, int D, int
 template <int D>
 static int launch_split(const FwdArgs &a, const SplitArgs &sp, hipStream_t st) {
   const int R = a.G * a.Sq;
-  const int ntile_r = (R + 127) / 128;
-  hipLaunchKernelGGL((fwd_bf16_kernel<D, 4, true>), dim3((unsigned)(ntile_r * sp.nsplit * a.Hkv * a.B)),
-                     dim3(256), 0, st, a, sp);
+  const int rc = launch_fwd_t<D, 4, true>(a, sp, st);
+  if (rc) return rc;
   constexpr int RPB = 256 / (D / 4);
   const int64_t rows = (int64_t)a.B * a.Hkv * R;
   hipLaunchKernelGGL(fwd_combine_kernel<D>, dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, a,
@@ -390,7 +395,7 @@ static int launch_split(const FwdArgs &a, const SplitArgs &sp, hipStream_t st) {
 int launch_fwd_kvcache_bf16(const FwdArgs &a, const SplitArgs &sp_in, int D, hipStream_t st) {
   SplitArgs sp = sp_in;
   int ns, tps;
-  plan_split(a.B, a.Sq, a.Sk, a.H, a.Hkv, &ns, &tps);
+  plan_split(a.B, a.Sq, a.Sk0, a.Sk, a.H, a.Hkv, &ns, &tps);
   if (ns <= 1) return launch_fwd_bf16(a, D, st);
   sp.nsplit = ns;
   sp.tiles_per_split = tps;

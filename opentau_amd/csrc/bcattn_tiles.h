@@ -1,0 +1,152 @@
+// LDS tiles of the MFMA kernels: 64 rows x D bf16, filled by buffer loads that
+// write LDS directly, read either as row operands (16-byte reads) or as
+// transposed operands (ds_read_b64_tr_b16), with one XOR swizzle that keeps both
+// kinds of read free of bank conflicts.
+#pragma once
+
+#include "bcattn_common.h"
+
+namespace bcattn {
+
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4_t;
+
+// A 64 x D tile.  Row r occupies bytes [r*2D, (r+1)*2D); inside the row the
+// 16-byte slot that holds columns 8L..8L+7 sits at slot L ^ swz(r).
+//
+// Row reads: 16 lanes read the same logical slot of 16 consecutive rows; swz is
+// a bijection of (r mod 16) [of (r/2 mod 8) for D=64, whose rows are 128 bytes],
+// so they land in 16 different slots = all 64 banks.
+// Transposed reads: 32 lanes read two adjacent slots of 4 consecutive rows (two
+// 16-lane groups, the second two slots further); swz>>1 takes 4 different
+// values on 4 consecutive rows, so the 8 slot pairs are again all 64 banks.
+template <int D>
+struct Tile {
+  static constexpr int kSlotsPerRow = D / 8;
+  static constexpr int kRowBytes = 2 * D;
+  static constexpr int kBytes = 64 * kRowBytes;
+  static constexpr int kSlots = 64 * kSlotsPerRow;
+
+  __device__ __forceinline__ static int swz(int r) {
+    if (D == 64) return (((r >> 1) & 1) << 2) | (((r >> 2) & 1) << 1) | ((r >> 3) & 1);
+    return ((r & 3) << 2) | ((r >> 2) & 3);
+  }
+  // Byte offset of logical slot L of row r.
+  __device__ __forceinline__ static int off(int r, int L) { return r * kRowBytes + 16 * (L ^ swz(r)); }
+};
+
+// Buffer descriptor over `bytes` bytes at p (loads past the end return zero), in
+// scalar registers.  Base and size are the same in every lane; reading them from
+// the first lane is what puts them in scalar registers.
+typedef i32x4 buf_rsrc_t;
+__device__ __forceinline__ buf_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
+  const uint64_t addr = reinterpret_cast<uint64_t>(p);
+  buf_rsrc_t r;
+  r[0] = __builtin_amdgcn_readfirstlane((int)(uint32_t)addr);
+  r[1] = __builtin_amdgcn_readfirstlane((int)((uint32_t)(addr >> 32) & 0xffffu));
+  r[2] = __builtin_amdgcn_readfirstlane((int)bytes);
+  r[3] = 0x00020000;  // raw buffer, 32-bit data format
+  return r;
+}
+
+// Byte address of an LDS location, as the hardware counts it.
+__device__ __forceinline__ uint32_t lds_addr(const void *p) {
+  return (uint32_t)(uintptr_t)((__attribute__((address_space(3))) const char *)p);
+}
+
+// Asynchronous global -> LDS copy, 16 (or 4) bytes per lane: lane l reads
+// base + voff + soff and writes LDS byte lds_base + 16*l (4*l).  Issued as
+// assembly so that the compiler does not order later LDS reads of the *other*
+// stage behind it; completion is awaited explicitly with wait_async_loads().
+__device__ __forceinline__ void dma16(buf_rsrc_t rsrc, uint32_t lds_base, uint32_t voff, uint32_t soff) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+      :
+      : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
+      : "memory", "m0");
+}
+__device__ __forceinline__ void dma4(buf_rsrc_t rsrc, uint32_t lds_base, uint32_t voff, uint32_t soff) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+      :
+      : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
+      : "memory", "m0");
+}
+
+// Per-thread source offsets of an asynchronous tile load.  The tile's kSlots
+// 16-byte slots are covered by kSlots/NT loads per thread; load x of wave w
+// fills the 64 consecutive LDS slots (x*NT + 64*w) .. +63, lane l the l-th, and
+// fetches the matching (row, logical slot) of the source.
+template <int D, int NT>
+struct TileLoad {
+  static constexpr int kLoads = Tile<D>::kSlots / NT;
+  static_assert(Tile<D>::kSlots % NT == 0, "tile slots must divide over the threads");
+  uint32_t voff[kLoads];
+
+  __device__ __forceinline__ void init(int tid, int64_t row_stride_elems) {
+#pragma unroll
+    for (int x = 0; x < kLoads; ++x) {
+      const int s = x * NT + tid;
+      const int row = s / Tile<D>::kSlotsPerRow, P = s % Tile<D>::kSlotsPerRow;
+      const int L = P ^ Tile<D>::swz(row);
+      voff[x] = (uint32_t)(row * row_stride_elems * 2 + L * 16);
+    }
+  }
+  // `tile` is the LDS tile base, `soff` the byte offset of the tile's first row.
+  __device__ __forceinline__ void issue(buf_rsrc_t rsrc, const char *tile, uint32_t soff, int wave) const {
+    const uint32_t base = __builtin_amdgcn_readfirstlane(lds_addr(tile) + 1024u * (uint32_t)wave);
+    const uint32_t so = __builtin_amdgcn_readfirstlane(soff);
+#pragma unroll
+    for (int x = 0; x < kLoads; ++x) dma16(rsrc, base + (uint32_t)(x * NT * 16), voff[x], so);
+  }
+};
+
+// 64 consecutive dwords -> LDS, one per lane (a whole wave must call it).
+__device__ __forceinline__ void load_row64_dwords(buf_rsrc_t rsrc, const void *dst, uint32_t soff, int lane) {
+  dma4(rsrc, __builtin_amdgcn_readfirstlane(lds_addr(dst)), (uint32_t)lane * 4,
+       __builtin_amdgcn_readfirstlane(soff));
+}
+
+__device__ __forceinline__ void wait_async_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// Row operand of a 32x32x16 product: row (rbase + lane%32), columns 16*ks + 8*(lane/32) .. +7.
+template <int D>
+__device__ __forceinline__ bf16x8 row_operand(const char *tile, int row, int ks, int hh) {
+  return *reinterpret_cast<const bf16x8 *>(tile + Tile<D>::off(row, 2 * ks + hh));
+}
+
+// Per-lane constants of the transposed operand reads.
+template <int D>
+struct TrLane {
+  int row_lo;   // 4*hh + (lane%16)/4 : row inside the 16-row group, first half
+  int slot_lo;  // logical slot of the lane's 4 columns inside a 32-column block
+  int byte;     // 0 or 8: which half of the slot
+  __device__ __forceinline__ void init(int lane) {
+    const int i = lane & 15, grp = (lane >> 4) & 1, hh = lane >> 5;
+    row_lo = 4 * hh + (i >> 2);
+    slot_lo = 2 * grp + ((i & 3) >> 1);
+    byte = 8 * (i & 1);
+  }
+};
+
+// Transposed operand: for output row d = 32*db + lane%32 the 8 sequence positions
+//   16*kk + 8*(e/4) + 4*(lane/32) + e%4,  e = 0..7
+// of a row-major tile (positions are tile rows), i.e. exactly the positions whose
+// values a lane holds in registers 8*half .. 8*half+7 of a 32x32 accumulator.
+// Two ds_read_b64_tr_b16: within 16 lanes, lane i receives, from the 8-byte rows
+// the 16 lanes point at, element (i%4) of rows 4e + i/4 -- a 4x16 transpose.
+template <int D>
+__device__ __forceinline__ bf16x8 tr_operand(const char *tile, const TrLane<D> &t, int kk, int db) {
+  const int r0 = 16 * kk + t.row_lo, r1 = r0 + 8;
+  const int L = 4 * db + t.slot_lo;
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (lds_s16x4_t *)(tile + Tile<D>::off(r0, L) + t.byte));
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (lds_s16x4_t *)(tile + Tile<D>::off(r1, L) + t.byte));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(bf16x8, both);
+}
+
+}  // namespace bcattn

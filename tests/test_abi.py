@@ -44,7 +44,9 @@ def test_workspace_queries_run_without_a_gpu():
     p.B, p.Sq, p.Sk0, p.Sk1, p.H, p.Hkv, p.D, p.dtype = 8, 50, 968, 50, 8, 1, 256, _loader.DTYPE_BF16
     fwd = lib.bcattn_fwd_workspace_bytes(ctypes.byref(p))
     kvc = lib.bcattn_fwd_kvcache_workspace_bytes(ctypes.byref(p))
-    assert fwd == 8 * 16 * 16  # 16 key tiles of 64 per sample, 16 bytes each
+    # 16 + 1 key tiles per sample (the two segments are tiled separately): a 16-byte summary
+    # and 64 merged ids per tile, each array rounded up to 256 bytes
+    assert fwd == (8 * 17 * 16 + 255) // 256 * 256 + 8 * 17 * 64 * 4
     assert kvc > fwd
     bp = _loader.BwdParams()
     bp.B, bp.Sq, bp.Sk, bp.H, bp.Hkv, bp.D = 2, 100, 130, 4, 2, 128

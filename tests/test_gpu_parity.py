@@ -321,7 +321,9 @@ def test_kvcache_equals_concat(b, sq, h, hkv, d, cross):
     o_split, l_split = fa.forward_raw(g(q), g(kc), g(vc), *gi, d**-0.5, g(kn), g(vn), kvcache=True)
     o_sq, l_sq = fa.forward_raw(g(q), g(k), g(v), *gi, d**-0.5)
     o_2seg, _ = fa.forward_raw(g(q), g(kc), g(vc), *gi, d**-0.5, g(kn), g(vn))
-    assert torch.equal(o_2seg, o_sq)  # two segments read in place == the concatenation
+    # two segments read in place == the concatenation (key tiles are cut per segment, so the
+    # summation order, and with it the last bit, may differ)
+    assert max_abs(o_2seg.float(), o_sq.float()) <= 2 * 2**-8 * float(ref.abs().max())
     assert_close_bf16(o_split.float().cpu(), ref, "split out")
     torch.testing.assert_close(l_split, l_sq, atol=1e-5, rtol=1e-5)
     assert max_abs(o_split.float(), o_sq.float()) <= 2 * 2**-8 * float(ref.abs().max())
