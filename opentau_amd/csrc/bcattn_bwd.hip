@@ -57,6 +57,12 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const BwdArgs a) {
   }
 }
 
+// LDS stages: three where they fit in the 160 KB of a CU, else two.
+template <int D>
+struct BwdStages {
+  static constexpr int value = D <= 128 ? 3 : 2;
+};
+
 // ---- dQ ------------------------------------------------------------------------
 template <int D, int NW>
 __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
@@ -64,6 +70,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   constexpr int NT = 64 * NW, BM = 32 * NW;
   constexpr int DK = D / 16, DB = D / 32;
   constexpr int STAGE = 2 * T::kBytes + 256;  // K tile, V tile, 64 key ids
+  constexpr int NS = BwdStages<D>::value;
 
   extern __shared__ __align__(1024) char smem[];
   __shared__ int red_s[2 * NW];
@@ -135,27 +142,28 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   vld.init(tid, a.v.ss);
   const uint32_t kstep = (uint32_t)(64 * a.k.ss * 2), vstep = (uint32_t)(64 * a.v.ss * 2);
 
-  // Next tile at or after t that some row of the workgroup can see, with its summary.
-  // (Summaries are read before a tile's asynchronous loads are issued: an ordinary
-  // load issued after them could only complete once they have.)
-  tile_summary_t sm_next = {0, 0, 0, 0};
-  auto next_needed = [&](int t) {
+  const_summary_t *ksum_s = scalar_view(ksum);
+  // First tile at or after t that some row of the workgroup can see, with its summary.
+  auto next_needed = [&](int t, tile_summary_t &sm) {
     while (t < nt) {
-      sm_next = ksum[t];
-      if (sm_next.x <= qmax_g) break;
+      sm = ksum_s[t];
+      if (sm.x <= qmax_g) break;
       ++t;
     }
-    sm_next = uniform_summary(sm_next);
-    return __builtin_amdgcn_readfirstlane(t);  // same in every lane; tell the compiler so
+    return t;
   };
-  auto issue = [&](int t, char *st) {
+  auto issue = [&](int t, auto stage_c) {
+    const char *st = smem + decltype(stage_c)::value * STAGE;
     kld.issue(krs, st, (uint32_t)t * kstep, wave);
     vld.issue(vrs, st + T::kBytes, (uint32_t)t * vstep, wave);
-    if (wave == 0) load_row64_dwords(idrs, st + 2 * T::kBytes, (uint32_t)t * 256, lane);
+    load_row64_dwords(idrs, st + 2 * T::kBytes, (uint32_t)t * 256, lane);  // every wave, same data
   };
+  constexpr int LPT = 2 * TileLoad<D, NT>::kLoads + 1;  // loads per tile and wave
 
-  TrLane<D> trl;
-  trl.init(lane);
+  RowAddr<D> rowa;
+  rowa.init(lane);
+  TrAddr<D> tra;
+  tra.init(lane);
 
   f32x16 dq[DB];
 #pragma unroll
@@ -164,8 +172,9 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
     for (int x = 0; x < 16; ++x) dq[db][x] = 0.f;
   const float c = a.scale * kLog2e;
 
-  auto compute = [&](const char *st, const tile_summary_t sm) {
+  auto compute = [&](auto stage_c, const tile_summary_t sm) {
     if (sm.x > qmax_w) return;  // wave-uniform: no row of this wave sees a key of the tile
+    const char *st = smem + decltype(stage_c)::value * STAGE;
     const char *Kt = st, *Vt = st + T::kBytes;
     const int *kb_s = reinterpret_cast<const int *>(st + 2 * T::kBytes);
     const bool needmask = !(sm.z != 0 && sm.y <= qmin_w);
@@ -180,8 +189,8 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
         bf16x8 fa[KB], fb[KB];
 #pragma unroll
         for (int ks = 0; ks < KB; ++ks) {
-          fa[ks] = row_operand<D>(Kt, 32 * mb + n, k0 + ks, hh);
-          fb[ks] = row_operand<D>(Vt, 32 * mb + n, k0 + ks, hh);
+          fa[ks] = rowa.read(Kt, 32 * mb, k0 + ks);
+          fb[ks] = rowa.read(Vt, 32 * mb, k0 + ks);
         }
 #pragma unroll
         for (int ks = 0; ks < KB; ++ks) {
@@ -208,7 +217,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
       for (int half = 0; half < 2; ++half) {
         bf16x8 ka[DB];
 #pragma unroll
-        for (int db = 0; db < DB; ++db) ka[db] = tr_operand<D>(Kt, trl, 2 * mb + half, db);
+        for (int db = 0; db < DB; ++db) ka[db] = tra.read(Kt, 2 * mb + half, db);
 #pragma unroll
         for (int db = 0; db < DB; ++db) dq[db] = mfma32(ka[db], dsb[half], dq[db]);
       }
@@ -216,19 +225,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   };
 
   // Two LDS stages: while tile t is being used, tile t+1 streams into the other one.
-  int t = next_needed(0);
-  int stage = 0;
-  if (t < nt) issue(t, smem);
-  while (t < nt) {
-    const tile_summary_t sm = sm_next;
-    const int tn = next_needed(t + 1);
-    wait_async_loads();
-    __syncthreads();
-    if (tn < nt) issue(tn, smem + (stage ^ 1) * STAGE);
-    compute(smem + stage * STAGE, sm);
-    t = tn;
-    stage ^= 1;
-  }
+  tile_pipeline<NS, LPT>(0, nt, next_needed, issue, compute);
 
   if (rowok) {
     bf16_t *optr = reinterpret_cast<bf16_t *>(a.dq) + b * a.dq_sb + (int64_t)i * a.dq_ss + h * a.dq_sh;
@@ -246,7 +243,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
 
 template <int D>
 constexpr size_t dq_smem_bytes() {
-  return 2 * (2 * (size_t)Tile<D>::kBytes + 256);
+  return BwdStages<D>::value * (2 * (size_t)Tile<D>::kBytes + 256);
 }
 
 // ---- dK / dV ---------------------------------------------------------------------
@@ -255,6 +252,7 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
   using T = Tile<D>;
   constexpr int DK = D / 16, DB = D / 32;
   constexpr int STAGE = 2 * T::kBytes + 3 * 256;  // Q tile, dO tile, lse2, delta, q ids
+  constexpr int NS = BwdStages<D>::value;
 
   extern __shared__ __align__(1024) char smem[];
   __shared__ int red_s[4];
@@ -313,30 +311,39 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
   gld.init(tid, a.d_o.ss);
   const uint32_t qstep = (uint32_t)(64 * a.q.ss * 2), gstep = (uint32_t)(64 * a.d_o.ss * 2);
 
-  tile_summary_t sm_next = {0, 0, 0, 0};
-  auto next_needed = [&](int it) {
+  const_summary_t *qsum_s = scalar_view(qsum);
+  // Iterations run over (query head of the group, query tile); first needed one at or after it.
+  auto next_needed = [&](int it, tile_summary_t &sm) {
     while (it < nit) {
-      sm_next = qsum[it % nqt];
-      if (sm_next.w > 0 && sm_next.y >= kmin_g) break;
+      sm = qsum_s[it % nqt];
+      if (sm.w > 0 && sm.y >= kmin_g) break;
       ++it;
     }
-    sm_next = uniform_summary(sm_next);
-    return __builtin_amdgcn_readfirstlane(it);  // same in every lane; tell the compiler so
+    return it;
   };
-  auto issue = [&](int it, char *st) {
+  auto issue = [&](int it, auto stage_c) {
+    const char *st = smem + decltype(stage_c)::value * STAGE;
     const int g = it / nqt, qt = it - g * nqt;
     const buf_rsrc_t qrs = make_rsrc(qb0 + (int64_t)g * a.q.sh, qbytes);
     const buf_rsrc_t grs = make_rsrc(gb0 + (int64_t)g * a.d_o.sh, gbytes);
     qld.issue(qrs, st, (uint32_t)qt * qstep, wave);
     gld.issue(grs, st + T::kBytes, (uint32_t)qt * gstep, wave);
-    char *aux = st + 2 * T::kBytes;
-    if (wave == 0) load_row64_dwords(lrs, aux, (uint32_t)(g * Sqp + qt * 64) * 4, lane);
-    if (wave == 1) load_row64_dwords(drs, aux + 256, (uint32_t)(g * Sqp + qt * 64) * 4, lane);
-    if (wave == 2) load_row64_dwords(irs, aux + 512, (uint32_t)(qt * 64) * 4, lane);
+    // one statistics row per wave (the fourth wave repeats the first one's)
+    const char *aux = st + 2 * T::kBytes;
+    const uint32_t srow = (uint32_t)(g * Sqp + qt * 64) * 4;
+    if (wave == 1)
+      load_row64_dwords(drs, aux + 256, srow, lane);
+    else if (wave == 2)
+      load_row64_dwords(irs, aux + 512, (uint32_t)(qt * 64) * 4, lane);
+    else
+      load_row64_dwords(lrs, aux, srow, lane);
   };
+  constexpr int LPT = 2 * TileLoad<D, 256>::kLoads + 1;  // loads per tile and wave
 
-  TrLane<D> trl;
-  trl.init(lane);
+  RowAddr<D> rowa;
+  rowa.init(lane);
+  TrAddr<D> tra;
+  tra.init(lane);
 
   f32x16 dk[DB], dv[DB];
 #pragma unroll
@@ -345,8 +352,9 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
     for (int x = 0; x < 16; ++x) dk[db][x] = 0.f, dv[db][x] = 0.f;
   const float c = a.scale * kLog2e;
 
-  auto compute = [&](const char *st, const tile_summary_t sm) {
+  auto compute = [&](auto stage_c, const tile_summary_t sm) {
     if (sm.y < kmin_w) return;  // wave-uniform: no key of this wave is seen by the tile
+    const char *st = smem + decltype(stage_c)::value * STAGE;
     const char *Qt = st, *Gt = st + T::kBytes;
     const float *lse_s = reinterpret_cast<const float *>(st + 2 * T::kBytes);
     const float *delta_s = lse_s + 64;
@@ -363,8 +371,8 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
         bf16x8 fa[KB], fb[KB];
 #pragma unroll
         for (int ks = 0; ks < KB; ++ks) {
-          fa[ks] = row_operand<D>(Qt, 32 * mb + n, k0 + ks, hh);
-          fb[ks] = row_operand<D>(Gt, 32 * mb + n, k0 + ks, hh);
+          fa[ks] = rowa.read(Qt, 32 * mb, k0 + ks);
+          fb[ks] = rowa.read(Gt, 32 * mb, k0 + ks);
         }
 #pragma unroll
         for (int ks = 0; ks < KB; ++ks) {
@@ -401,8 +409,8 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
           bf16x8 ga[DBB], qa[DBB];
 #pragma unroll
           for (int db = 0; db < DBB; ++db) {
-            ga[db] = tr_operand<D>(Gt, trl, 2 * mb + half, d0 + db);
-            qa[db] = tr_operand<D>(Qt, trl, 2 * mb + half, d0 + db);
+            ga[db] = tra.read(Gt, 2 * mb + half, d0 + db);
+            qa[db] = tra.read(Qt, 2 * mb + half, d0 + db);
           }
 #pragma unroll
           for (int db = 0; db < DBB; ++db) {
@@ -414,19 +422,7 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
     }
   };
 
-  int it = next_needed(0);
-  int stage = 0;
-  if (it < nit) issue(it, smem);
-  while (it < nit) {
-    const tile_summary_t sm = sm_next;
-    const int itn = next_needed(it + 1);
-    wait_async_loads();
-    __syncthreads();
-    if (itn < nit) issue(itn, smem + (stage ^ 1) * STAGE);
-    compute(smem + stage * STAGE, sm);
-    it = itn;
-    stage ^= 1;
-  }
+  tile_pipeline<NS, LPT>(0, nit, next_needed, issue, compute);
 
   if (jok) {
     bf16_t *dkp = reinterpret_cast<bf16_t *>(a.dk) + b * a.dk_sb + (int64_t)j * a.dk_ss + hk * a.dk_sh;
@@ -449,7 +445,7 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
 
 template <int D>
 constexpr size_t dkv_smem_bytes() {
-  return 2 * (2 * (size_t)Tile<D>::kBytes + 3 * 256);
+  return BwdStages<D>::value * (2 * (size_t)Tile<D>::kBytes + 3 * 256);
 }
 
 template <int D, int NWQ>

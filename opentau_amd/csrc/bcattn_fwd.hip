@@ -19,6 +19,12 @@ namespace bcattn {
 // writes its unnormalised fp32 partial (O, running max, sum) and
 // `fwd_combine_kernel` merges them.  This is what lets a handful of
 // (batch, kv head) problems with few query rows fill the chip.
+// LDS stages: three where they fit in the 160 KB of a CU, else two.
+template <int D>
+struct FwdStages {
+  static constexpr int value = D <= 128 ? 3 : 2;
+};
+
 template <int D, int NW, bool SPLIT>
 __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, const SplitArgs sp) {
   using T = Tile<D>;
@@ -27,6 +33,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   constexpr int DK = D / 16;    // contraction steps of K Q^T
   constexpr int DB = D / 32;    // 32-row blocks of O^T
   constexpr int STAGE = 2 * T::kBytes + 256;  // K tile, V tile, 64 key ids
+  constexpr int NS = FwdStages<D>::value;
 
   extern __shared__ __align__(1024) char smem[];
   __shared__ int red_s[2 * NW];
@@ -104,20 +111,18 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   k1ld.init(tid, a.k1.ss);
   v1ld.init(tid, a.v1.ss);
 
-  // Next tile at or after t that some row of the workgroup can see, with its summary.
-  // (Summaries are read before a tile's asynchronous loads are issued: an ordinary
-  // load issued after them could only complete once they have.)
-  tile_summary_t sm_next = {0, 0, 0, 0};
-  auto next_needed = [&](int t) {
+  const_summary_t *ksum_s = scalar_view(ksum);
+  // First tile at or after t that some row of the workgroup can see, with its summary.
+  auto next_needed = [&](int t, tile_summary_t &sm) {
     while (t < nt) {
-      sm_next = ksum[t];
-      if (sm_next.x <= qmax_g) break;
+      sm = ksum_s[t];
+      if (sm.x <= qmax_g) break;
       ++t;
     }
-    sm_next = uniform_summary(sm_next);
-    return __builtin_amdgcn_readfirstlane(t);  // same in every lane; tell the compiler so
+    return t;
   };
-  auto issue = [&](int t, char *st) {
+  auto issue = [&](int t, auto stage_c) {
+    const char *st = smem + decltype(stage_c)::value * STAGE;
     if (t < nt0) {
       k0ld.issue(k0rs, st, (uint32_t)(t * 64 * a.k0.ss * 2), wave);
       v0ld.issue(v0rs, st + T::kBytes, (uint32_t)(t * 64 * a.v0.ss * 2), wave);
@@ -125,11 +130,14 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
       k1ld.issue(k1rs, st, (uint32_t)((t - nt0) * 64 * a.k1.ss * 2), wave);
       v1ld.issue(v1rs, st + T::kBytes, (uint32_t)((t - nt0) * 64 * a.v1.ss * 2), wave);
     }
-    if (wave == 0) load_row64_dwords(idrs, st + 2 * T::kBytes, (uint32_t)t * 256, lane);
+    load_row64_dwords(idrs, st + 2 * T::kBytes, (uint32_t)t * 256, lane);  // every wave, same data
   };
+  constexpr int LPT = 2 * TileLoad<D, NT>::kLoads + 1;  // loads per tile and wave
 
-  TrLane<D> trl;
-  trl.init(lane);
+  RowAddr<D> rowa;
+  rowa.init(lane);
+  TrAddr<D> tra;
+  tra.init(lane);
 
   // ---- running state ---------------------------------------------------------
   f32x16 o[DB];
@@ -141,8 +149,9 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   float l = 0.f;        // this lane half's share of the running sum
   const float c = a.scale * kLog2e;
 
-  auto compute = [&](const char *st, const tile_summary_t sm) {
+  auto compute = [&](auto stage_c, const tile_summary_t sm) {
     if (sm.x > qmax_w) return;  // wave-uniform: no row of this wave sees a key of the tile
+    const char *st = smem + decltype(stage_c)::value * STAGE;
     const char *Kt = st, *Vt = st + T::kBytes;
     const int *kb_s = reinterpret_cast<const int *>(st + 2 * T::kBytes);
     // Two independent accumulator chains (the two 32-key halves) are interleaved:
@@ -159,8 +168,8 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
         bf16x8 ka0[KB], ka1[KB];
 #pragma unroll
         for (int ks = 0; ks < KB; ++ks) {
-          ka0[ks] = row_operand<D>(Kt, n, k0 + ks, hh);
-          ka1[ks] = row_operand<D>(Kt, 32 + n, k0 + ks, hh);
+          ka0[ks] = rowa.read(Kt, 0, k0 + ks);
+          ka1[ks] = rowa.read(Kt, 32, k0 + ks);
         }
 #pragma unroll
         for (int ks = 0; ks < KB; ++ks) {
@@ -218,7 +227,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
       for (int d0 = 0; d0 < DB; d0 += DBB) {
         bf16x8 va[DBB];
 #pragma unroll
-        for (int db = 0; db < DBB; ++db) va[db] = tr_operand<D>(Vt, trl, kk, d0 + db);
+        for (int db = 0; db < DBB; ++db) va[db] = tra.read(Vt, kk, d0 + db);
 #pragma unroll
         for (int db = 0; db < DBB; ++db) o[d0 + db] = mfma32(va[db], pb[kk], o[d0 + db]);
       }
@@ -226,19 +235,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   };
 
   // Two LDS stages: while tile t is being used, tile t+1 streams into the other one.
-  int t = next_needed(t_first);
-  int stage = 0;
-  if (t < nt) issue(t, smem);
-  while (t < nt) {
-    const tile_summary_t sm = sm_next;
-    const int tn = next_needed(t + 1);
-    wait_async_loads();
-    __syncthreads();
-    if (tn < nt) issue(tn, smem + (stage ^ 1) * STAGE);
-    compute(smem + stage * STAGE, sm);
-    t = tn;
-    stage ^= 1;
-  }
+  tile_pipeline<NS, LPT>(t_first, nt, next_needed, issue, compute);
 
   // ---- epilogue ----------------------------------------------------------------
   l += swap32(l);
@@ -284,7 +281,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
 
 template <int D>
 constexpr size_t fwd_smem_bytes() {
-  return 2 * (2 * (size_t)Tile<D>::kBytes + 256);
+  return FwdStages<D>::value * (2 * (size_t)Tile<D>::kBytes + 256);
 }
 
 // Merge the per-split partials: one thread per (packed row, 4 head_dim columns).

@@ -110,23 +110,25 @@ __device__ __forceinline__ void load_row64_dwords(buf_rsrc_t rsrc, const void *d
 
 __device__ __forceinline__ void wait_async_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
-// Row operand of a 32x32x16 product: row (rbase + lane%32), columns 16*ks + 8*(lane/32) .. +7.
-template <int D>
-__device__ __forceinline__ bf16x8 row_operand(const char *tile, int row, int ks, int hh) {
-  return *reinterpret_cast<const bf16x8 *>(tile + Tile<D>::off(row, 2 * ks + hh));
-}
+// ---------------------------------------------------------------------------
+// Operand reads.  The swizzle makes a read address a per-lane XOR pattern rather
+// than base + constant, so each lane computes its offsets once, before the main
+// loop; in the loop an address is (precomputed lane offset) + (compile-time
+// tile / stage / block constant), which folds into the instruction's immediate.
+// ---------------------------------------------------------------------------
 
-// Per-lane constants of the transposed operand reads.
+// Row operand of a 32x32x16 product: row (rbase + lane%32), columns
+// 16*ks + 8*(lane/32) .. +7.  rbase must be a multiple of 16 rows.
 template <int D>
-struct TrLane {
-  int row_lo;   // 4*hh + (lane%16)/4 : row inside the 16-row group, first half
-  int slot_lo;  // logical slot of the lane's 4 columns inside a 32-column block
-  int byte;     // 0 or 8: which half of the slot
+struct RowAddr {
+  int a[D / 16];
   __device__ __forceinline__ void init(int lane) {
-    const int i = lane & 15, grp = (lane >> 4) & 1, hh = lane >> 5;
-    row_lo = 4 * hh + (i >> 2);
-    slot_lo = 2 * grp + ((i & 3) >> 1);
-    byte = 8 * (i & 1);
+    const int n = lane & 31, hh = lane >> 5;
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) a[ks] = Tile<D>::off(n, 2 * ks + hh);
+  }
+  __device__ __forceinline__ bf16x8 read(const char *tile, int rbase, int ks) const {
+    return *reinterpret_cast<const bf16x8 *>(tile + rbase * Tile<D>::kRowBytes + a[ks]);
   }
 };
 
@@ -135,18 +137,105 @@ struct TrLane {
 // of a row-major tile (positions are tile rows), i.e. exactly the positions whose
 // values a lane holds in registers 8*half .. 8*half+7 of a 32x32 accumulator.
 // Two ds_read_b64_tr_b16: within 16 lanes, lane i receives, from the 8-byte rows
-// the 16 lanes point at, element (i%4) of rows 4e + i/4 -- a 4x16 transpose.
+// the 16 lanes point at, element (i%4) of rows 4e + i/4 -- a 4x16 transpose.  So
+// lane i of a group points at row 4*(lane/32) + i/4 (+8 for the second read),
+// columns 32*db + 16*(group%2) + 4*(i%4) .. +3.
 template <int D>
-__device__ __forceinline__ bf16x8 tr_operand(const char *tile, const TrLane<D> &t, int kk, int db) {
-  const int r0 = 16 * kk + t.row_lo, r1 = r0 + 8;
-  const int L = 4 * db + t.slot_lo;
-  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-      (lds_s16x4_t *)(tile + Tile<D>::off(r0, L) + t.byte));
-  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-      (lds_s16x4_t *)(tile + Tile<D>::off(r1, L) + t.byte));
-  typedef short s16x8 __attribute__((ext_vector_type(8)));
-  const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-  return __builtin_bit_cast(bf16x8, both);
+struct TrAddr {
+  int lo[D / 32], hi[D / 32];
+  __device__ __forceinline__ void init(int lane) {
+    const int i = lane & 15, grp = (lane >> 4) & 1, hh = lane >> 5;
+    const int row = 4 * hh + (i >> 2);
+    const int slot = 2 * grp + ((i & 3) >> 1);
+    const int byte = 8 * (i & 1);
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db) {
+      lo[db] = Tile<D>::off(row, 4 * db + slot) + byte;
+      hi[db] = Tile<D>::off(row + 8, 4 * db + slot) + byte;
+    }
+  }
+  __device__ __forceinline__ bf16x8 read(const char *tile, int kk, int db) const {
+    const char *base = tile + 16 * kk * Tile<D>::kRowBytes;
+    const s16x4 l = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t *)(base + lo[db]));
+    const s16x4 h = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t *)(base + hi[db]));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    const s16x8 both = __builtin_shufflevector(l, h, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, both);
+  }
+};
+
+// Compile-time stage index, so that stage offsets fold into immediates.
+template <int S>
+struct StageC {
+  static constexpr int value = S;
+};
+
+// Tile summaries are read with scalar loads (uniform address, memory that no
+// kernel writes while this one runs): they come back through the scalar cache
+// and do not queue behind the asynchronous tile loads.
+typedef const __attribute__((address_space(4))) tile_summary_t const_summary_t;
+__device__ __forceinline__ const_summary_t *scalar_view(const tile_summary_t *p) {
+  return (const_summary_t *)reinterpret_cast<uintptr_t>(p);
+}
+
+// Wait until at most N of this wave's asynchronous loads are still in flight.
+template <int N>
+__device__ __forceinline__ void wait_async_loads_but() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+// Workgroup barrier without the fence of __syncthreads(): the tile data it orders
+// was already awaited by each wave (wait_async_loads*), and a fence would drain
+// the loads that are meant to stay in flight.
+__device__ __forceinline__ void tile_barrier() { asm volatile("s_barrier" ::: "memory"); }
+
+// Walk the needed tiles of [first, end) with NS LDS stages, i.e. NS-1 tiles of
+// asynchronous loads in flight while one is computed on.
+//   next(t, sm)        first needed tile >= t (or end) and its summary
+//   issue(t, StageC)   start the loads of tile t into that stage; every wave must
+//                      issue exactly LPT loads
+//   compute(StageC, sm)
+// The loop is written out over the stages so that every LDS address inside
+// compute() is a lane offset plus a compile-time constant.
+template <int NS, int LPT, class Next, class Issue, class Compute>
+__device__ __forceinline__ void tile_pipeline(int first, int end, Next next, Issue issue, Compute compute) {
+  static_assert(NS == 2 || NS == 3, "two or three stages");
+  tile_summary_t s0 = {0, 0, 0, 0}, s1 = s0, s2 = s0;
+  int t0 = next(first, s0);
+  if (t0 >= end) return;
+  issue(t0, StageC<0>{});
+  int t1 = end, t2 = end;
+  if (NS == 3) {
+    t1 = next(t0 + 1, s1);
+    if (t1 < end) issue(t1, StageC<1>{});
+  }
+  auto step = [&](auto sc) {
+    constexpr int S = decltype(sc)::value;
+    if (NS == 2) {
+      t1 = next(t0 + 1, s1);
+      wait_async_loads_but<0>();
+      tile_barrier();
+      if (t1 < end) issue(t1, StageC<(S + 1) % 2>{});
+      compute(sc, s0);
+      t0 = t1, s0 = s1;
+    } else {
+      t2 = t1 < end ? next(t1 + 1, s2) : end;
+      if (t1 < end)
+        wait_async_loads_but<LPT>();  // the newer tile may still be in flight
+      else
+        wait_async_loads_but<0>();
+      tile_barrier();
+      if (t2 < end) issue(t2, StageC<(S + 2) % 3>{});
+      compute(sc, s0);
+      t0 = t1, s0 = s1, t1 = t2, s1 = s2;
+    }
+    return t0 >= end;
+  };
+  for (;;) {
+    if (step(StageC<0>{})) break;
+    if (step(StageC<1>{})) break;
+    if (NS == 3)
+      if (step(StageC<2>{})) break;
+  }
 }
 
 }  // namespace bcattn
