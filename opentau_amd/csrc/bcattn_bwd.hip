@@ -81,7 +81,9 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
 
   const int R = a.G * a.Sq;
   const int ntile_r = (R + BM - 1) / BM;
-  int bid = blockIdx.x;
+  const int nitems = ntile_r * a.Hkv * a.B;
+  int bid = xcd_item(blockIdx.x, nitems);
+  if (bid >= nitems) return;
   const int tile = __builtin_amdgcn_readfirstlane(bid % ntile_r);
   bid /= ntile_r;
   // (division results live in vector registers; say that they are uniform)
@@ -174,6 +176,9 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
 
   auto compute = [&](auto stage_c, const tile_summary_t sm) {
     if (sm.x > qmax_w) return;  // wave-uniform: no row of this wave sees a key of the tile
+#ifdef IGLP
+    __builtin_amdgcn_iglp_opt(IGLP);
+#endif
     const char *st = smem + decltype(stage_c)::value * STAGE;
     const char *Kt = st, *Vt = st + T::kBytes;
     const int *kb_s = reinterpret_cast<const int *>(st + 2 * T::kBytes);
@@ -263,7 +268,9 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
 
   const int Sk = a.Sk, Sq = a.Sq, Sqp = a.Sq_pad;
   const int nkt = (Sk + 127) / 128;
-  int bid = blockIdx.x;
+  const int nitems = nkt * a.Hkv * a.B;
+  int bid = xcd_item(blockIdx.x, nitems);
+  if (bid >= nitems) return;
   const int kt = __builtin_amdgcn_readfirstlane(bid % nkt);
   bid /= nkt;
   // (division results live in vector registers; say that they are uniform)
@@ -352,74 +359,136 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
     for (int x = 0; x < 16; ++x) dk[db][x] = 0.f, dv[db][x] = 0.f;
   const float c = a.scale * kLog2e;
 
-  auto compute = [&](auto stage_c, const tile_summary_t sm) {
-    if (sm.y < kmin_w) return;  // wave-uniform: no key of this wave is seen by the tile
+  // One query tile, software-pipelined inside the wave so that the vector ALU work
+  // of one 32-query half runs in the shadow of the other half's matrix products:
+  //   A0 | A1 + softmax0 | C0 + softmax1 | C1
+  // A(mb): S = Q K^T and dP = dO V^T of queries 32mb.. (row operands from LDS)
+  // softmax(mb): P = exp2(c S - log2e LSE), dS = P o (dP - delta), packed to bf16
+  // C(mb): dV^T += dO^T P, dK^T += Q^T dS (transposed operands from LDS)
+  // The scheduler is given the interleaving explicitly (sched_group_barrier:
+  // 0x008 matrix, 0x100 LDS read, 0x002 vector ALU); MASKED is a compile-time copy
+  // of "some pair of this tile may be masked", so the common case carries no
+  // compare/select at all.
+  auto compute_t = [&](auto stage_c, auto masked_c) {
+    constexpr bool MASKED = decltype(masked_c)::value != 0;
     const char *st = smem + decltype(stage_c)::value * STAGE;
     const char *Qt = st, *Gt = st + T::kBytes;
     const float *lse_s = reinterpret_cast<const float *>(st + 2 * T::kBytes);
     const float *delta_s = lse_s + 64;
     const int *qb_s = reinterpret_cast<const int *>(delta_s + 64);
-    const bool needmask = !(sm.z != 0 && allk_w != 0 && kmax_w <= sm.x);
+    f32x16 s[2], dp[2];
+    bf16x8 pb[2][2], dsb[2][2];
+
+    auto phase_a = [&](int mb) {
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb) {
-      f32x16 s, dp;
+      for (int x = 0; x < 16; ++x) s[mb][x] = 0.f, dp[mb][x] = 0.f;
 #pragma unroll
-      for (int x = 0; x < 16; ++x) s[x] = 0.f, dp[x] = 0.f;
-      constexpr int KB = DK < 4 ? DK : 4;
-#pragma unroll
-      for (int k0 = 0; k0 < DK; k0 += KB) {
-        bf16x8 fa[KB], fb[KB];
-#pragma unroll
-        for (int ks = 0; ks < KB; ++ks) {
-          fa[ks] = rowa.read(Qt, 32 * mb, k0 + ks);
-          fb[ks] = rowa.read(Gt, 32 * mb, k0 + ks);
-        }
-#pragma unroll
-        for (int ks = 0; ks < KB; ++ks) {
-          s = mfma32(fa[ks], kf[k0 + ks], s);
-          dp = mfma32(fb[ks], vf[k0 + ks], dp);
-        }
+      for (int ks = 0; ks < DK; ++ks) {
+        const bf16x8 fa = rowa.read(Qt, 32 * mb, ks);
+        const bf16x8 fb = rowa.read(Gt, 32 * mb, ks);
+        s[mb] = mfma32(fa, kf[ks], s[mb]);
+        dp[mb] = mfma32(fb, vf[ks], dp[mb]);
       }
-      float p[16], ds[16];
-#pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        const int q0 = 32 * mb + 8 * r4 + 4 * hh;
-        const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lse_s + q0);
-        const f32x4 del4 = *reinterpret_cast<const f32x4 *>(delta_s + q0);
-        i32x4 qb4 = {0, 0, 0, 0};
-        if (needmask) qb4 = *reinterpret_cast<const i32x4 *>(qb_s + q0);
-#pragma unroll
-        for (int x = 0; x < 4; ++x) {
-          float pv = fast_exp2(s[4 * r4 + x] * c - lse4[x]);
-          if (needmask && kb > qb4[x]) pv = 0.f;
-          p[4 * r4 + x] = pv;
-          ds[4 * r4 + x] = pv * (dp[4 * r4 + x] - del4[x]);
-        }
-      }
-      bf16x8 pb[2], dsb[2];
-      pb[0] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
-      pb[1] = pack8(p[8], p[9], p[10], p[11], p[12], p[13], p[14], p[15]);
-      dsb[0] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
-      dsb[1] = pack8(ds[8], ds[9], ds[10], ds[11], ds[12], ds[13], ds[14], ds[15]);
+    };
+    auto softmax = [&](int mb) {
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
-        constexpr int DBB = DB < 4 ? DB : 4;
+        float p[8], ds[8];
 #pragma unroll
-        for (int d0 = 0; d0 < DB; d0 += DBB) {
-          bf16x8 ga[DBB], qa[DBB];
+        for (int r2 = 0; r2 < 2; ++r2) {
+          const int r4 = 2 * half + r2;
+          const int q0 = 32 * mb + 8 * r4 + 4 * hh;
+          const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lse_s + q0);
+          const f32x4 del4 = *reinterpret_cast<const f32x4 *>(delta_s + q0);
+          i32x4 qb4 = {0, 0, 0, 0};
+          if (MASKED) qb4 = *reinterpret_cast<const i32x4 *>(qb_s + q0);
 #pragma unroll
-          for (int db = 0; db < DBB; ++db) {
-            ga[db] = tra.read(Gt, 2 * mb + half, d0 + db);
-            qa[db] = tra.read(Qt, 2 * mb + half, d0 + db);
-          }
-#pragma unroll
-          for (int db = 0; db < DBB; ++db) {
-            dv[d0 + db] = mfma32(ga[db], pb[half], dv[d0 + db]);
-            dk[d0 + db] = mfma32(qa[db], dsb[half], dk[d0 + db]);
+          for (int x = 0; x < 4; ++x) {
+            float pv = fast_exp2(s[mb][4 * r4 + x] * c - lse4[x]);
+            if (MASKED && kb > qb4[x]) pv = 0.f;
+            p[4 * r2 + x] = pv;
+            ds[4 * r2 + x] = pv * (dp[mb][4 * r4 + x] - del4[x]);
           }
         }
+        pb[mb][half] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
+        dsb[mb][half] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
+      }
+    };
+    auto phase_c = [&](int mb) {
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const bf16x8 ga = tra.read(Gt, 2 * mb + half, db);
+          const bf16x8 qa = tra.read(Qt, 2 * mb + half, db);
+          dv[db] = mfma32(ga, pb[mb][half], dv[db]);
+          dk[db] = mfma32(qa, dsb[mb][half], dk[db]);
+        }
+    };
+    constexpr int NA = 2 * DK;   // products (= row-operand reads) of one A phase
+    constexpr int NC = 4 * DB;   // products of one C phase (two LDS reads each)
+    constexpr int VA = MASKED ? 9 : 7;  // vector ALU instructions per product, about
+
+    phase_a(0);
+    {
+      constexpr int kAhead = NA < 6 ? NA : 6;
+      __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+      for (int x = 0; x < NA - kAhead; ++x) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    phase_a(1);
+    softmax(0);
+    {
+      constexpr int kAhead = NA < 4 ? NA : 4;
+      __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+      for (int x = 0; x < NA; ++x) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // next operand + statistics reads
+        __builtin_amdgcn_sched_group_barrier(0x002, VA, 0);
       }
     }
+    __builtin_amdgcn_sched_barrier(0);
+
+    phase_c(0);
+    softmax(1);
+    {
+      constexpr int kAhead = NC < 4 ? NC : 4;
+      __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
+#pragma unroll
+      for (int x = 0; x < NC; ++x) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, VA, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    phase_c(1);
+    {
+      constexpr int kAhead = NC < 4 ? NC : 4;
+      __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
+#pragma unroll
+      for (int x = 0; x < NC - kAhead; ++x) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto compute = [&](auto stage_c, const tile_summary_t sm) {
+    if (sm.y < kmin_w) return;  // wave-uniform: no key of this wave is seen by the tile
+    if (sm.z != 0 && allk_w != 0 && kmax_w <= sm.x)
+      compute_t(stage_c, StageC<0>{});  // every pair of the tile attends
+    else
+      compute_t(stage_c, StageC<1>{});
   };
 
   tile_pipeline<NS, LPT>(0, nit, next_needed, issue, compute);
@@ -463,12 +532,12 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
   if (a.stages & BCATTN_BWD_DQ) {
     const int R = a.G * a.Sq;
     const int ntile_r = (R + 32 * NWQ - 1) / (32 * NWQ);
-    hipLaunchKernelGGL((bwd_dq_kernel<D, NWQ>), dim3((unsigned)(ntile_r * a.Hkv * a.B)), dim3(64 * NWQ),
+    hipLaunchKernelGGL((bwd_dq_kernel<D, NWQ>), dim3(xcd_grid((unsigned)(ntile_r * a.Hkv * a.B))), dim3(64 * NWQ),
                        dq_smem_bytes<D>(), st, a);
   }
   if (a.stages & BCATTN_BWD_DKV) {
     const int nkt = (a.Sk + 127) / 128;
-    hipLaunchKernelGGL((bwd_dkv_kernel<D>), dim3((unsigned)(nkt * a.Hkv * a.B)), dim3(256),
+    hipLaunchKernelGGL((bwd_dkv_kernel<D>), dim3(xcd_grid((unsigned)(nkt * a.Hkv * a.B))), dim3(256),
                        dkv_smem_bytes<D>(), st, a);
   }
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;

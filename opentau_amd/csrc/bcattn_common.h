@@ -98,6 +98,20 @@ __device__ __forceinline__ bf16x8 pack8(float a0, float a1, float a2, float a3, 
   return r;
 }
 
+// Workgroup -> work item map that keeps neighbours on one XCD.  The hardware
+// hands consecutive workgroup ids to the 8 XCDs in turn, each with its own L2;
+// work items that stream the same K/V (or Q/dO) are consecutive, so item
+//   (id % 8) * ceil(n/8) + id / 8
+// puts a run of consecutive items on one XCD, where they share what they stream
+// through that L2.  The grid is rounded up to 8*ceil(n/8); ids that map past n
+// have nothing to do.
+constexpr int kXcds = 8;
+__host__ __device__ __forceinline__ unsigned xcd_grid(unsigned n) { return kXcds * ((n + kXcds - 1) / kXcds); }
+__device__ __forceinline__ int xcd_item(unsigned id, unsigned n) {
+  const unsigned chunk = (n + kXcds - 1) / kXcds;
+  return (int)((id % kXcds) * chunk + id / kXcds);
+}
+
 // ---------------------------------------------------------------------------
 // LDS layouts.
 //

@@ -44,7 +44,9 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
 
   const int R = a.G * a.Sq;
   const int ntile_r = (R + BM - 1) / BM;
-  int bid = blockIdx.x;
+  const int nitems = ntile_r * (SPLIT ? sp.nsplit : 1) * a.Hkv * a.B;
+  int bid = xcd_item(blockIdx.x, nitems);
+  if (bid >= nitems) return;
   const int tile = __builtin_amdgcn_readfirstlane(bid % ntile_r);
   bid /= ntile_r;
   const int split = SPLIT ? __builtin_amdgcn_readfirstlane(bid % sp.nsplit) : 0;
@@ -151,6 +153,9 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
 
   auto compute = [&](auto stage_c, const tile_summary_t sm) {
     if (sm.x > qmax_w) return;  // wave-uniform: no row of this wave sees a key of the tile
+#ifdef IGLP
+    __builtin_amdgcn_iglp_opt(IGLP);
+#endif
     const char *st = smem + decltype(stage_c)::value * STAGE;
     const char *Kt = st, *Vt = st + T::kBytes;
     const int *kb_s = reinterpret_cast<const int *>(st + 2 * T::kBytes);
@@ -335,7 +340,7 @@ static int launch_fwd_t(const FwdArgs &a, const SplitArgs &sp, hipStream_t st) {
   const int R = a.G * a.Sq;
   const int ntile_r = (R + 32 * NW - 1) / (32 * NW);
   hipLaunchKernelGGL((fwd_bf16_kernel<D, NW, SPLIT>),
-                     dim3((unsigned)(ntile_r * (SPLIT ? sp.nsplit : 1) * a.Hkv * a.B)), dim3(64 * NW),
+                     dim3(xcd_grid((unsigned)(ntile_r * (SPLIT ? sp.nsplit : 1) * a.Hkv * a.B))), dim3(64 * NW),
                      fwd_smem_bytes<D>(), st, a, sp);
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
 }

@@ -3,7 +3,8 @@
 Counterpart of ``src/opentau/policies/flash_attn_cuda/_loader.py:42-103``: lazy,
 once per process, lock-guarded, with ``is_available()`` / ``load_error()`` and an
 environment kill-switch.  Unlike the reference nothing is compiled at run time:
-the library is built ahead of time (``make -C opentau_amd/csrc``) and there is
+the library is built ahead of time (``make -C opentau_amd/csrc``; ``OPENTAU_FLASH_HIP_LIB``
+names another build of it) and there is
 **no fallback** — when the library or a GPU is missing, calls raise.
 """
 
@@ -142,9 +143,10 @@ def load_library() -> ctypes.CDLL:
     """
     if os.environ.get("OPENTAU_DISABLE_FLASH_HIP", "0") == "1":
         raise RuntimeError("flash_hip disabled via OPENTAU_DISABLE_FLASH_HIP=1")
-    if not LIB_PATH.exists():
-        raise RuntimeError(f"{LIB_PATH} not built; run `make -C {CSRC}`")
-    lib = ctypes.CDLL(str(LIB_PATH))
+    path = Path(os.environ.get("OPENTAU_FLASH_HIP_LIB", str(LIB_PATH)))
+    if not path.exists():
+        raise RuntimeError(f"{path} not built; run `make -C {CSRC}`")
+    lib = ctypes.CDLL(str(path))
     missing = [s for s in EXPORTS if not hasattr(lib, s)]
     if missing:
         raise RuntimeError(f"{LIB_PATH} lacks symbols: {missing}")
