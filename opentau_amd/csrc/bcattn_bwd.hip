@@ -252,22 +252,30 @@ constexpr size_t dq_smem_bytes() {
 }
 
 // ---- dK / dV ---------------------------------------------------------------------
-template <int D>
-__global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
+// MODE selects what a launch produces: both gradients (one pass, needs K and V
+// fragments plus both accumulators in registers), or dV alone / dK alone (two
+// launches that each recompute S; this is what fits the register file at
+// head_dim 256, and at 128 it lets two waves share a SIMD).
+constexpr int kModeBoth = 0, kModeDV = 1, kModeDK = 2;
+
+template <int D, int NW, int MODE>
+__global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   using T = Tile<D>;
+  constexpr bool WANT_DV = MODE != kModeDK, WANT_DK = MODE != kModeDV;
+  constexpr int NT = 64 * NW, BK = 32 * NW;
   constexpr int DK = D / 16, DB = D / 32;
   constexpr int STAGE = 2 * T::kBytes + 3 * 256;  // Q tile, dO tile, lse2, delta, q ids
   constexpr int NS = BwdStages<D>::value;
 
   extern __shared__ __align__(1024) char smem[];
-  __shared__ int red_s[4];
+  __shared__ int red_s[NW];
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
 
   const int Sk = a.Sk, Sq = a.Sq, Sqp = a.Sq_pad;
-  const int nkt = (Sk + 127) / 128;
+  const int nkt = (Sk + BK - 1) / BK;
   const int nitems = nkt * a.Hkv * a.B;
   int bid = xcd_item(blockIdx.x, nitems);
   if (bid >= nitems) return;
@@ -278,7 +286,7 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
   const int b = __builtin_amdgcn_readfirstlane(bid / a.Hkv);
 
   // ---- this lane's key -----------------------------------------------------
-  const int j = kt * 128 + wave * 32 + n;
+  const int j = kt * BK + wave * 32 + n;
   const bool jok = j < Sk;
   const int jj = jok ? j : Sk - 1;
   const bool kv = jok && a.k_valid[(int64_t)b * Sk + jj] != 0;
@@ -287,18 +295,20 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
       reinterpret_cast<const bf16_t *>(a.k.ptr) + b * a.k.sb + (int64_t)jj * a.k.ss + hk * a.k.sh;
   const bf16_t *vptr =
       reinterpret_cast<const bf16_t *>(a.v.ptr) + b * a.v.sb + (int64_t)jj * a.v.ss + hk * a.v.sh;
-  bf16x8 kf[DK], vf[DK];
+  bf16x8 kf[DK], vf[WANT_DK ? DK : 1];
 #pragma unroll
   for (int ks = 0; ks < DK; ++ks) {
     kf[ks] = *reinterpret_cast<const bf16x8 *>(kptr + 16 * ks + 8 * hh);
-    vf[ks] = *reinterpret_cast<const bf16x8 *>(vptr + 16 * ks + 8 * hh);
+    if (WANT_DK) vf[ks] = *reinterpret_cast<const bf16x8 *>(vptr + 16 * ks + 8 * hh);
   }
   const int kmin_w = wave_min_i(kb);
   const int kmax_w = wave_max_i(kv ? kb : kIntMin);
   const int allk_w = wave_min_i(kv ? 1 : 0);
   if (lane == 0) red_s[wave] = kmin_w;
   __syncthreads();
-  const int kmin_g = min(min(red_s[0], red_s[1]), min(red_s[2], red_s[3]));
+  int kmin_g = kIntMax;
+#pragma unroll
+  for (int x = 0; x < NW; ++x) kmin_g = min(kmin_g, red_s[x]);
 
   const int nqt = Sqp / 64;
   const tile_summary_t *qsum = a.qsum + (int64_t)b * nqt;
@@ -313,7 +323,7 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
   const buf_rsrc_t lrs = make_rsrc(a.lse2 + stat0, (uint32_t)(a.G * Sqp * 4));
   const buf_rsrc_t drs = make_rsrc(a.delta + stat0, (uint32_t)(a.G * Sqp * 4));
   const buf_rsrc_t irs = make_rsrc(a.qbm + (int64_t)b * Sqp, (uint32_t)(Sqp * 4));
-  TileLoad<D, 256> qld, gld;
+  TileLoad<D, NT> qld, gld;
   qld.init(tid, a.q.ss);
   gld.init(tid, a.d_o.ss);
   const uint32_t qstep = (uint32_t)(64 * a.q.ss * 2), gstep = (uint32_t)(64 * a.d_o.ss * 2);
@@ -335,28 +345,31 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
     const buf_rsrc_t grs = make_rsrc(gb0 + (int64_t)g * a.d_o.sh, gbytes);
     qld.issue(qrs, st, (uint32_t)qt * qstep, wave);
     gld.issue(grs, st + T::kBytes, (uint32_t)qt * gstep, wave);
-    // one statistics row per wave (the fourth wave repeats the first one's)
+    // one statistics row per wave (further waves repeat one)
     const char *aux = st + 2 * T::kBytes;
     const uint32_t srow = (uint32_t)(g * Sqp + qt * 64) * 4;
-    if (wave == 1)
+    if (wave % 3 == 1)
       load_row64_dwords(drs, aux + 256, srow, lane);
-    else if (wave == 2)
+    else if (wave % 3 == 2)
       load_row64_dwords(irs, aux + 512, (uint32_t)(qt * 64) * 4, lane);
     else
       load_row64_dwords(lrs, aux, srow, lane);
   };
-  constexpr int LPT = 2 * TileLoad<D, 256>::kLoads + 1;  // loads per tile and wave
+  constexpr int LPT = 2 * TileLoad<D, NT>::kLoads + 1;  // loads per tile and wave
 
   RowAddr<D> rowa;
   rowa.init(lane);
   TrAddr<D> tra;
   tra.init(lane);
 
-  f32x16 dk[DB], dv[DB];
+  f32x16 dk[WANT_DK ? DB : 1], dv[WANT_DV ? DB : 1];
 #pragma unroll
   for (int db = 0; db < DB; ++db)
 #pragma unroll
-    for (int x = 0; x < 16; ++x) dk[db][x] = 0.f, dv[db][x] = 0.f;
+    for (int x = 0; x < 16; ++x) {
+      if (WANT_DK) dk[db][x] = 0.f;
+      if (WANT_DV) dv[db][x] = 0.f;
+    }
   const float c = a.scale * kLog2e;
 
   // One query tile, software-pipelined inside the wave so that the vector ALU work
@@ -376,18 +389,19 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
     const float *lse_s = reinterpret_cast<const float *>(st + 2 * T::kBytes);
     const float *delta_s = lse_s + 64;
     const int *qb_s = reinterpret_cast<const int *>(delta_s + 64);
-    f32x16 s[2], dp[2];
+    f32x16 s[2], dp[WANT_DK ? 2 : 1];
     bf16x8 pb[2][2], dsb[2][2];
 
     auto phase_a = [&](int mb) {
 #pragma unroll
-      for (int x = 0; x < 16; ++x) s[mb][x] = 0.f, dp[mb][x] = 0.f;
+      for (int x = 0; x < 16; ++x) {
+        s[mb][x] = 0.f;
+        if (WANT_DK) dp[mb][x] = 0.f;
+      }
 #pragma unroll
       for (int ks = 0; ks < DK; ++ks) {
-        const bf16x8 fa = rowa.read(Qt, 32 * mb, ks);
-        const bf16x8 fb = rowa.read(Gt, 32 * mb, ks);
-        s[mb] = mfma32(fa, kf[ks], s[mb]);
-        dp[mb] = mfma32(fb, vf[ks], dp[mb]);
+        s[mb] = mfma32(rowa.read(Qt, 32 * mb, ks), kf[ks], s[mb]);
+        if (WANT_DK) dp[mb] = mfma32(rowa.read(Gt, 32 * mb, ks), vf[ks], dp[mb]);
       }
     };
     auto softmax = [&](int mb) {
@@ -399,7 +413,8 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
           const int r4 = 2 * half + r2;
           const int q0 = 32 * mb + 8 * r4 + 4 * hh;
           const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lse_s + q0);
-          const f32x4 del4 = *reinterpret_cast<const f32x4 *>(delta_s + q0);
+          f32x4 del4 = {0.f, 0.f, 0.f, 0.f};
+          if (WANT_DK) del4 = *reinterpret_cast<const f32x4 *>(delta_s + q0);
           i32x4 qb4 = {0, 0, 0, 0};
           if (MASKED) qb4 = *reinterpret_cast<const i32x4 *>(qb_s + q0);
 #pragma unroll
@@ -407,11 +422,11 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
             float pv = fast_exp2(s[mb][4 * r4 + x] * c - lse4[x]);
             if (MASKED && kb > qb4[x]) pv = 0.f;
             p[4 * r2 + x] = pv;
-            ds[4 * r2 + x] = pv * (dp[mb][4 * r4 + x] - del4[x]);
+            if (WANT_DK) ds[4 * r2 + x] = pv * (dp[mb][4 * r4 + x] - del4[x]);
           }
         }
-        pb[mb][half] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
-        dsb[mb][half] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
+        if (WANT_DV) pb[mb][half] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
+        if (WANT_DK) dsb[mb][half] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
       }
     };
     auto phase_c = [&](int mb) {
@@ -419,15 +434,14 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
       for (int half = 0; half < 2; ++half)
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-          const bf16x8 ga = tra.read(Gt, 2 * mb + half, db);
-          const bf16x8 qa = tra.read(Qt, 2 * mb + half, db);
-          dv[db] = mfma32(ga, pb[mb][half], dv[db]);
-          dk[db] = mfma32(qa, dsb[mb][half], dk[db]);
+          if (WANT_DV) dv[db] = mfma32(tra.read(Gt, 2 * mb + half, db), pb[mb][half], dv[db]);
+          if (WANT_DK) dk[db] = mfma32(tra.read(Qt, 2 * mb + half, db), dsb[mb][half], dk[db]);
         }
     };
-    constexpr int NA = 2 * DK;   // products (= row-operand reads) of one A phase
-    constexpr int NC = 4 * DB;   // products of one C phase (two LDS reads each)
-    constexpr int VA = MASKED ? 9 : 7;  // vector ALU instructions per product, about
+    constexpr int PER = (WANT_DV ? 1 : 0) + (WANT_DK ? 1 : 0);
+    constexpr int NA = PER == 2 ? 2 * DK : (WANT_DK ? 2 * DK : DK);  // products of one A phase
+    constexpr int NC = 2 * DB * PER;                                  // products of one C phase
+    constexpr int VA = (MASKED ? 9 : 7) * 16 / (NA < NC ? NA : NC) + 1;  // vector ALU instr. per product
 
     phase_a(0);
     {
@@ -503,11 +517,11 @@ __global__ __launch_bounds__(256) void bwd_dkv_kernel(const BwdArgs a) {
         bf16x4 wk, wv;
 #pragma unroll
         for (int x = 0; x < 4; ++x) {
-          wk[x] = (bf16_t)(dk[db][4 * r4 + x] * a.scale);
-          wv[x] = (bf16_t)dv[db][4 * r4 + x];
+          if (WANT_DK) wk[x] = (bf16_t)(dk[db][4 * r4 + x] * a.scale);
+          if (WANT_DV) wv[x] = (bf16_t)dv[db][4 * r4 + x];
         }
-        *reinterpret_cast<bf16x4 *>(dkp + 32 * db + 8 * r4 + 4 * hh) = wk;
-        *reinterpret_cast<bf16x4 *>(dvp + 32 * db + 8 * r4 + 4 * hh) = wv;
+        if (WANT_DK) *reinterpret_cast<bf16x4 *>(dkp + 32 * db + 8 * r4 + 4 * hh) = wk;
+        if (WANT_DV) *reinterpret_cast<bf16x4 *>(dvp + 32 * db + 8 * r4 + 4 * hh) = wv;
       }
   }
 }
@@ -517,12 +531,23 @@ constexpr size_t dkv_smem_bytes() {
   return BwdStages<D>::value * (2 * (size_t)Tile<D>::kBytes + 3 * 256);
 }
 
-template <int D, int NWQ>
+template <int D, int NW, int MODE>
+static int launch_dkv(const BwdArgs &a, hipStream_t st) {
+  if (hipFuncSetAttribute(reinterpret_cast<const void *>(&bwd_dkv_kernel<D, NW, MODE>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)dkv_smem_bytes<D>()) != hipSuccess)
+    return BCATTN_ERR_LAUNCH;
+  const int nkt = (a.Sk + 32 * NW - 1) / (32 * NW);
+  hipLaunchKernelGGL((bwd_dkv_kernel<D, NW, MODE>), dim3(xcd_grid((unsigned)(nkt * a.Hkv * a.B))),
+                     dim3(64 * NW), dkv_smem_bytes<D>(), st, a);
+  return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
+}
+
+// NWQ: waves of the dQ kernel; NWK, SPLIT: waves of the dK/dV kernel and whether it
+// runs as two launches (dV, then dK).
+template <int D, int NWQ, int NWK, bool SPLIT>
 static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
   if (hipFuncSetAttribute(reinterpret_cast<const void *>(&bwd_dq_kernel<D, NWQ>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)dq_smem_bytes<D>()) != hipSuccess ||
-      hipFuncSetAttribute(reinterpret_cast<const void *>(&bwd_dkv_kernel<D>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)dkv_smem_bytes<D>()) != hipSuccess)
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)dq_smem_bytes<D>()) != hipSuccess)
     return BCATTN_ERR_LAUNCH;
   if (a.stages & BCATTN_BWD_DELTA) {
     constexpr int RPB = 256 / (D / 8);
@@ -536,9 +561,12 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
                        dq_smem_bytes<D>(), st, a);
   }
   if (a.stages & BCATTN_BWD_DKV) {
-    const int nkt = (a.Sk + 127) / 128;
-    hipLaunchKernelGGL((bwd_dkv_kernel<D>), dim3(xcd_grid((unsigned)(nkt * a.Hkv * a.B))), dim3(256),
-                       dkv_smem_bytes<D>(), st, a);
+    int rc;
+    if (SPLIT) {
+      if ((rc = launch_dkv<D, NWK, kModeDV>(a, st)) || (rc = launch_dkv<D, NWK, kModeDK>(a, st))) return rc;
+    } else if ((rc = launch_dkv<D, NWK, kModeBoth>(a, st))) {
+      return rc;
+    }
   }
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
 }
@@ -547,11 +575,15 @@ int launch_bwd_bf16(const BwdArgs &a, int D, hipStream_t st) {
   const int R = a.G * a.Sq;
   switch (D) {
     case 64:
-      return launch_bwd_d<64, 4>(a, st);
+      return launch_bwd_d<64, 4, 4, false>(a, st);
     case 128:
-      return R >= 1024 ? launch_bwd_d<128, 8>(a, st) : launch_bwd_d<128, 4>(a, st);
+#ifdef DKV128_SPLIT
+      return R >= 1024 ? launch_bwd_d<128, 8, 8, true>(a, st) : launch_bwd_d<128, 4, 4, false>(a, st);
+#else
+      return R >= 1024 ? launch_bwd_d<128, 8, 4, false>(a, st) : launch_bwd_d<128, 4, 4, false>(a, st);
+#endif
     case 256:
-      return launch_bwd_d<256, 4>(a, st);
+      return launch_bwd_d<256, 4, 4, true>(a, st);
     default:
       return BCATTN_ERR_UNSUPPORTED;
   }
