@@ -35,6 +35,9 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-denoise", action="store_true", help="skip the pi0.5 denoise leg")
     ap.add_argument("--workload", default="c5", choices=["c3", "c4", "c5"])
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
+                    help="only run a plain device copy of MIB MiB a few times (reference for the "
+                         "FETCH_SIZE / WRITE_SIZE counters) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
@@ -52,6 +55,16 @@ def main() -> int:
         return 1
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.copy_calibration:
+        n = args.copy_calibration << 20
+        src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes": n, "launches": 5}))
+        return 0
 
     w = make_workload(args.workload)
     pairs = w.pairs()
