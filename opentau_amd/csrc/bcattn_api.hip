@@ -249,8 +249,9 @@ int bcattn_fwd_kvcache(const bcattn_fwd_params *p, void *stream) {
   s.tiles_per_split = 0;
   kvcache_workspace_bytes(a.B, a.Sq, a.Sk0, a.Sk, a.H, a.Hkv, p->D, &s.nsplit);
   const size_t R = (size_t)a.G * a.Sq;
-  s.part_o = reinterpret_cast<float *>(ws);
-  s.part_ml = s.part_o + (size_t)a.B * a.Hkv * s.nsplit * R * p->D;
+  const size_t rows = (size_t)a.B * a.Hkv * s.nsplit * ((R + kSplitRows - 1) / kSplitRows) * kSplitRows;
+  s.part_ml = reinterpret_cast<float *>(ws);
+  s.part_o = reinterpret_cast<part_t *>(ws + split_ml_bytes(rows));
   rc = launch_fwd_kvcache_bf16(a, s, p->D, st);
   if (rc) return fail(rc, "kvcache forward launch failed (D=%d)", p->D);
   return BCATTN_OK;

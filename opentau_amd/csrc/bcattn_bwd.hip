@@ -533,8 +533,7 @@ constexpr size_t dkv_smem_bytes() {
 
 template <int D, int NW, int MODE>
 static int launch_dkv(const BwdArgs &a, hipStream_t st) {
-  if (hipFuncSetAttribute(reinterpret_cast<const void *>(&bwd_dkv_kernel<D, NW, MODE>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)dkv_smem_bytes<D>()) != hipSuccess)
+  if (!allow_dynamic_lds<&bwd_dkv_kernel<D, NW, MODE>>((int)dkv_smem_bytes<D>()))
     return BCATTN_ERR_LAUNCH;
   const int nkt = (a.Sk + 32 * NW - 1) / (32 * NW);
   hipLaunchKernelGGL((bwd_dkv_kernel<D, NW, MODE>), dim3(xcd_grid((unsigned)(nkt * a.Hkv * a.B))),
@@ -546,8 +545,7 @@ static int launch_dkv(const BwdArgs &a, hipStream_t st) {
 // runs as two launches (dV, then dK).
 template <int D, int NWQ, int NWK, bool SPLIT>
 static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
-  if (hipFuncSetAttribute(reinterpret_cast<const void *>(&bwd_dq_kernel<D, NWQ>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)dq_smem_bytes<D>()) != hipSuccess)
+  if (!allow_dynamic_lds<&bwd_dq_kernel<D, NWQ>>((int)dq_smem_bytes<D>()))
     return BCATTN_ERR_LAUNCH;
   if (a.stages & BCATTN_BWD_DELTA) {
     constexpr int RPB = 256 / (D / 8);

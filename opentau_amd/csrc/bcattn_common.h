@@ -2,6 +2,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <stdint.h>
 
 #include "bcattn.h"
@@ -217,6 +218,22 @@ struct BwdArgs {
   int stages;  // bit set of bcattn_bwd_stage, never 0 here
 };
 
+// Lets a kernel use more than 64 KB of dynamic LDS.  The attribute is per device, so a
+// bit per device remembers where it is already set and launches skip the runtime call.
+template <auto Kernel>
+inline bool allow_dynamic_lds(int bytes) {
+  static std::atomic<uint64_t> done{0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  const uint64_t bit = dev < 64 ? (uint64_t)1 << dev : 0;
+  if (bit && (done.load(std::memory_order_acquire) & bit)) return true;
+  if (hipFuncSetAttribute(reinterpret_cast<const void *>(Kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                          bytes) != hipSuccess)
+    return false;
+  done.fetch_or(bit, std::memory_order_release);
+  return true;
+}
+
 // kernel launchers, one translation unit each
 // Tile summaries and merged ids of a sequence given as two segments (n0 rows, then S - n0).
 int launch_summary(const int32_t *blk, const uint8_t *valid, int B, int n0, int S, int fill,
@@ -226,9 +243,27 @@ int launch_fwd_f32(const FwdArgs &a, int D, hipStream_t st);
 int launch_bwd_bf16(const BwdArgs &a, int D, hipStream_t st);
 int launch_bwd_f32(const BwdArgs &a, int D, hipStream_t st);
 
+// Split-key partials of the KV-cached forward.  A work item is (batch, kv head, split,
+// row tile of kSplitRows packed rows); its head_dim accumulators are stored in the order
+// the lanes hold them.
+#ifndef BCATTN_SPLIT_TARGET
+#define BCATTN_SPLIT_TARGET 256
+#endif
+#ifdef BCATTN_PART_BF16
+typedef bf16_t part_t;   // partials normalised by their own sum, so |value| <= max |v|
+typedef bf16x4 part4_t;
+constexpr bool kPartNormalized = true;
+#else
+typedef float part_t;
+typedef f32x4 part4_t;
+constexpr bool kPartNormalized = false;
+#endif
+constexpr int kSplitRows = 128;
+constexpr int kSplitTarget = BCATTN_SPLIT_TARGET;  // workgroups to aim for: one per CU, each holds most of a CU's LDS
+inline size_t split_ml_bytes(size_t rows) { return (rows * 2 * sizeof(float) + 255) & ~(size_t)255; }
 struct SplitArgs {
-  float *part_o;   // (B, Hkv, nsplit, R, D) fp32, R = G*Sq
-  float *part_ml;  // (B, Hkv, nsplit, R, 2) fp32: running max (raw scores), sum
+  part_t *part_o;  // (B, Hkv, nsplit, row tiles, kSplitRows * D)
+  float *part_ml;  // (B, Hkv, nsplit, row tiles, kSplitRows, 2): running max (raw scores), sum
   int nsplit;
   int tiles_per_split;  // 64-key tiles per split
 };

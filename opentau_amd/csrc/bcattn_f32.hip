@@ -151,8 +151,7 @@ static size_t fwd_f32_smem(int D) {
 
 int launch_fwd_f32(const FwdArgs &a, int D, hipStream_t st) {
   const size_t smem = fwd_f32_smem(D);
-  if (hipFuncSetAttribute(reinterpret_cast<const void *>(&fwd_f32_kernel),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)fwd_f32_smem(256)) != hipSuccess)
+  if (!allow_dynamic_lds<&fwd_f32_kernel>((int)fwd_f32_smem(256)))
     return BCATTN_ERR_LAUNCH;
   hipLaunchKernelGGL(fwd_f32_kernel, dim3((a.Sq + F_BR - 1) / F_BR, a.H, a.B), dim3(256), smem, st, a, D);
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
@@ -388,10 +387,8 @@ static size_t dkv_f32_smem(int D) {
 }
 
 int launch_bwd_f32(const BwdArgs &a, int D, hipStream_t st) {
-  if (hipFuncSetAttribute(reinterpret_cast<const void *>(&bwd_dq_f32_kernel),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)dq_f32_smem(256)) != hipSuccess ||
-      hipFuncSetAttribute(reinterpret_cast<const void *>(&bwd_dkv_f32_kernel),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)dkv_f32_smem(256)) != hipSuccess)
+  if (!allow_dynamic_lds<&bwd_dq_f32_kernel>((int)dq_f32_smem(256)) ||
+      !allow_dynamic_lds<&bwd_dkv_f32_kernel>((int)dkv_f32_smem(256)))
     return BCATTN_ERR_LAUNCH;
   const int64_t rows = (int64_t)a.B * a.Sq * a.H;
   if (a.stages & BCATTN_BWD_DELTA)

@@ -24,6 +24,11 @@ template <int D>
 struct FwdStages {
   static constexpr int value = D <= 128 ? 3 : 2;
 };
+// A split workgroup keeps every stage it has room for in flight from its first instruction.
+template <int D>
+struct SplitStages {
+  static constexpr int value = D <= 128 ? 4 : 2;
+};
 
 template <int D, int NW, bool SPLIT>
 __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, const SplitArgs sp) {
@@ -33,11 +38,10 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   constexpr int DK = D / 16;    // contraction steps of K Q^T
   constexpr int DB = D / 32;    // 32-row blocks of O^T
   constexpr int STAGE = 2 * T::kBytes + 256;  // K tile, V tile, 64 key ids
-  constexpr int NS = FwdStages<D>::value;
+  constexpr int NS = SPLIT ? SplitStages<D>::value : FwdStages<D>::value;
 
   extern __shared__ __align__(1024) char smem[];
   __shared__ int red_s[2 * NW];
-
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
@@ -55,6 +59,56 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   const int hk = __builtin_amdgcn_readfirstlane(bid % a.Hkv);
   const int b = __builtin_amdgcn_readfirstlane(bid / a.Hkv);
 
+  // Key tiles never straddle the two key segments: tiles [0, nt0) cover segment 0,
+  // tiles [nt0, nt0+nt1) segment 1, each padded (zero rows, invalid ids) at its end.
+  const int nt0 = (a.Sk0 + 63) / 64;
+  const int nt_all = nt0 + (a.Sk - a.Sk0 + 63) / 64;
+  const int t_first = SPLIT ? split * sp.tiles_per_split : 0;
+  const tile_summary_t *ksum = a.ksum + (int64_t)b * nt_all;
+
+  const bf16_t *k0b = reinterpret_cast<const bf16_t *>(a.k0.ptr) + b * a.k0.sb + hk * a.k0.sh;
+  const bf16_t *v0b = reinterpret_cast<const bf16_t *>(a.v0.ptr) + b * a.v0.sb + hk * a.v0.sh;
+  const bf16_t *k1b = reinterpret_cast<const bf16_t *>(a.k1.ptr) + b * a.k1.sb + hk * a.k1.sh;
+  const bf16_t *v1b = reinterpret_cast<const bf16_t *>(a.v1.ptr) + b * a.v1.sb + hk * a.v1.sh;
+  const int n0 = a.Sk0 > 0 ? a.Sk0 : 1, n1 = a.Sk - a.Sk0 > 0 ? a.Sk - a.Sk0 : 1;
+  const buf_rsrc_t k0rs = make_rsrc(k0b, (uint32_t)(((int64_t)(n0 - 1) * a.k0.ss + D) * 2));
+  const buf_rsrc_t v0rs = make_rsrc(v0b, (uint32_t)(((int64_t)(n0 - 1) * a.v0.ss + D) * 2));
+  const buf_rsrc_t k1rs = make_rsrc(k1b, (uint32_t)(((int64_t)(n1 - 1) * a.k1.ss + D) * 2));
+  const buf_rsrc_t v1rs = make_rsrc(v1b, (uint32_t)(((int64_t)(n1 - 1) * a.v1.ss + D) * 2));
+  const buf_rsrc_t idrs =
+      make_rsrc(a.kbm + (int64_t)b * nt_all * 64, (uint32_t)(nt_all * 64 * 4));
+  TileLoad<D, NT> k0ld, v0ld, k1ld, v1ld;
+  k0ld.init(tid, a.k0.ss);
+  v0ld.init(tid, a.v0.ss);
+  k1ld.init(tid, a.k1.ss);
+  v1ld.init(tid, a.v1.ss);
+
+  auto issue = [&](int t, auto stage_c) {
+    const char *st = smem + decltype(stage_c)::value * STAGE;
+    if (t < nt0) {
+      k0ld.issue(k0rs, st, (uint32_t)(t * 64 * a.k0.ss * 2), wave);
+      v0ld.issue(v0rs, st + T::kBytes, (uint32_t)(t * 64 * a.v0.ss * 2), wave);
+    } else {
+      k1ld.issue(k1rs, st, (uint32_t)((t - nt0) * 64 * a.k1.ss * 2), wave);
+      v1ld.issue(v1rs, st + T::kBytes, (uint32_t)((t - nt0) * 64 * a.v1.ss * 2), wave);
+    }
+    load_row64_dwords(idrs, st + 2 * T::kBytes, (uint32_t)t * 256, lane);  // every wave, same data
+  };
+  constexpr int LPT = 2 * TileLoad<D, NT>::kLoads + 1;  // loads per tile and wave
+
+  // A split workgroup has only a few tiles, so its start-up latency counts: its first
+  // tiles are requested before anything is known about the rows (compute() skips a
+  // tile that no row turns out to see).
+  const int t_last = SPLIT ? min(nt_all, t_first + sp.tiles_per_split) : nt_all;
+  if (SPLIT) {
+    if (t_first < t_last) issue(t_first, StageC<0>{});
+    if (t_first + 1 < t_last) issue(t_first + 1, StageC<1>{});
+    if constexpr (NS >= 3)
+      if (t_first + 2 < t_last) issue(t_first + 2, StageC<2>{});
+    if constexpr (NS >= 4)
+      if (t_first + 3 < t_last) issue(t_first + 3, StageC<3>{});
+  }
+
   // ---- this lane's query row ------------------------------------------------
   const int r = tile * BM + wave * 32 + n;
   const bool rowok = r < R;
@@ -62,8 +116,11 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   const int g = rr / a.Sq;
   const int i = rr - g * a.Sq;
   const int h = hk * a.G + g;
-  const bool qv = rowok && a.q_valid[(int64_t)b * a.Sq + i] != 0;
-  const int qb = qv ? a.q_blk[(int64_t)b * a.Sq + i] : kIntMin;
+  // both loads are unconditional so that they are in flight together
+  const uint8_t qv_raw = a.q_valid[(int64_t)b * a.Sq + i];
+  const int qb_raw = a.q_blk[(int64_t)b * a.Sq + i];
+  const bool qv = rowok && qv_raw != 0;
+  const int qb = qv ? qb_raw : kIntMin;
 
   const bf16_t *qptr =
       reinterpret_cast<const bf16_t *>(a.q.ptr) + b * a.q.sb + (int64_t)i * a.q.ss + h * a.q.sh;
@@ -88,31 +145,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
     any_g |= red_s[NW + x];
   }
 
-  // Key tiles never straddle the two key segments: tiles [0, nt0) cover segment 0,
-  // tiles [nt0, nt0+nt1) segment 1, each padded (zero rows, invalid ids) at its end.
-  const int nt0 = (a.Sk0 + 63) / 64;
-  const int nt_all = nt0 + (a.Sk - a.Sk0 + 63) / 64;
-  const int t_first = SPLIT ? split * sp.tiles_per_split : 0;
-  const int nt = !any_g ? 0 : (SPLIT ? min(nt_all, t_first + sp.tiles_per_split) : nt_all);
-  const tile_summary_t *ksum = a.ksum + (int64_t)b * nt_all;
-
-  const bf16_t *k0b = reinterpret_cast<const bf16_t *>(a.k0.ptr) + b * a.k0.sb + hk * a.k0.sh;
-  const bf16_t *v0b = reinterpret_cast<const bf16_t *>(a.v0.ptr) + b * a.v0.sb + hk * a.v0.sh;
-  const bf16_t *k1b = reinterpret_cast<const bf16_t *>(a.k1.ptr) + b * a.k1.sb + hk * a.k1.sh;
-  const bf16_t *v1b = reinterpret_cast<const bf16_t *>(a.v1.ptr) + b * a.v1.sb + hk * a.v1.sh;
-  const int n0 = a.Sk0 > 0 ? a.Sk0 : 1, n1 = a.Sk - a.Sk0 > 0 ? a.Sk - a.Sk0 : 1;
-  const buf_rsrc_t k0rs = make_rsrc(k0b, (uint32_t)(((int64_t)(n0 - 1) * a.k0.ss + D) * 2));
-  const buf_rsrc_t v0rs = make_rsrc(v0b, (uint32_t)(((int64_t)(n0 - 1) * a.v0.ss + D) * 2));
-  const buf_rsrc_t k1rs = make_rsrc(k1b, (uint32_t)(((int64_t)(n1 - 1) * a.k1.ss + D) * 2));
-  const buf_rsrc_t v1rs = make_rsrc(v1b, (uint32_t)(((int64_t)(n1 - 1) * a.v1.ss + D) * 2));
-  const buf_rsrc_t idrs =
-      make_rsrc(a.kbm + (int64_t)b * nt_all * 64, (uint32_t)(nt_all * 64 * 4));
-  TileLoad<D, NT> k0ld, v0ld, k1ld, v1ld;
-  k0ld.init(tid, a.k0.ss);
-  v0ld.init(tid, a.v0.ss);
-  k1ld.init(tid, a.k1.ss);
-  v1ld.init(tid, a.v1.ss);
-
+  const int nt = !any_g ? 0 : t_last;
   const_summary_t *ksum_s = scalar_view(ksum);
   // First tile at or after t that some row of the workgroup can see, with its summary.
   auto next_needed = [&](int t, tile_summary_t &sm) {
@@ -123,19 +156,6 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
     }
     return t;
   };
-  auto issue = [&](int t, auto stage_c) {
-    const char *st = smem + decltype(stage_c)::value * STAGE;
-    if (t < nt0) {
-      k0ld.issue(k0rs, st, (uint32_t)(t * 64 * a.k0.ss * 2), wave);
-      v0ld.issue(v0rs, st + T::kBytes, (uint32_t)(t * 64 * a.v0.ss * 2), wave);
-    } else {
-      k1ld.issue(k1rs, st, (uint32_t)((t - nt0) * 64 * a.k1.ss * 2), wave);
-      v1ld.issue(v1rs, st + T::kBytes, (uint32_t)((t - nt0) * 64 * a.v1.ss * 2), wave);
-    }
-    load_row64_dwords(idrs, st + 2 * T::kBytes, (uint32_t)t * 256, lane);  // every wave, same data
-  };
-  constexpr int LPT = 2 * TileLoad<D, NT>::kLoads + 1;  // loads per tile and wave
-
   RowAddr<D> rowa;
   rowa.init(lane);
   TrAddr<D> tra;
@@ -239,31 +259,46 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
     }
   };
 
-  // Two LDS stages: while tile t is being used, tile t+1 streams into the other one.
-  tile_pipeline<NS, LPT>(t_first, nt, next_needed, issue, compute);
+  if constexpr (SPLIT) {
+    // the summary of the next tile is fetched while this one is computed
+    tile_summary_t sm_next = ksum_s[min(t_first, nt_all - 1)];
+    auto compute_t = [&](auto stage_c, int t) {
+      const tile_summary_t sm = sm_next;
+      sm_next = ksum_s[min(t + 1, nt_all - 1)];
+      compute(stage_c, sm);
+    };
+    tile_burst<NS, LPT>(t_first, nt, issue, compute_t);
+    wait_async_loads_but<0>();  // the early requests, if no row of the workgroup is valid
+  } else {
+    // While tile t is being used, the next needed tile(s) stream into the other stage(s).
+    tile_pipeline<NS, LPT>(t_first, nt, next_needed, issue, compute);
+  }
 
   // ---- epilogue ----------------------------------------------------------------
   l += swap32(l);
   if (SPLIT) {
-    if (rowok) {
-      const int64_t prow = (((int64_t)b * a.Hkv + hk) * sp.nsplit + split) * R + r;
-      if (hh == 0) {
-        f32x2 ml;
-        ml[0] = qv ? m : -INFINITY;
-        ml[1] = qv ? l : 0.f;
-        *reinterpret_cast<f32x2 *>(sp.part_ml + 2 * prow) = ml;
-      }
-      float *po = sp.part_o + prow * D;
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-          f32x4 w;
-#pragma unroll
-          for (int x = 0; x < 4; ++x) w[x] = o[db][4 * r4 + x];
-          *reinterpret_cast<f32x4 *>(po + 32 * db + 8 * r4 + 4 * hh) = w;
-        }
+    // Partials stay in accumulator order (register-major, lane-minor): every store
+    // instruction writes 64 consecutive vectors.  Padding rows are written too
+    // (weight zero), so the merge needs no row test on its loads.
+    const int64_t item = (((int64_t)b * a.Hkv + hk) * sp.nsplit + split) * ntile_r + tile;
+    const bool has = qv && l > 0.f;
+    if (hh == 0) {
+      f32x2 ml;
+      ml[0] = has ? m : -INFINITY;
+      ml[1] = has ? l : 0.f;
+      *reinterpret_cast<f32x2 *>(sp.part_ml + 2 * (item * BM + wave * 32 + n)) = ml;
     }
+    part_t *po = sp.part_o + item * (BM * D) + (int64_t)wave * (32 * D) + 4 * lane;
+    const float pinv = kPartNormalized ? (has ? 1.f / l : 0.f) : 1.f;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        part4_t w;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) w[x] = (part_t)(o[db][4 * r4 + x] * pinv);
+        *reinterpret_cast<part4_t *>(po + (db * 4 + r4) * 256) = w;
+      }
     return;
   }
   const bool has = qv && l > 0.f;
@@ -284,41 +319,67 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   }
 }
 
-template <int D>
+template <int D, bool SPLIT>
 constexpr size_t fwd_smem_bytes() {
-  return FwdStages<D>::value * (2 * (size_t)Tile<D>::kBytes + 256);
+  return (SPLIT ? SplitStages<D>::value : FwdStages<D>::value) * (2 * (size_t)Tile<D>::kBytes + 256);
 }
 
-// Merge the per-split partials: one thread per (packed row, 4 head_dim columns).
-template <int D>
+// Merge the per-split partials.  A thread owns the same (wave, head_dim block, register
+// quad, lane) slot the split kernel's lanes wrote, so its loads are consecutive across
+// the wave; blockIdx.x = (batch, kv head, row tile), blockIdx.y = (wave, head_dim block).
+template <int D, int NW>
 __global__ __launch_bounds__(256) void fwd_combine_kernel(const FwdArgs a, const SplitArgs sp) {
-  constexpr int TPR = D / 4;
+  constexpr int DB = D / 32, BM = 32 * NW;
   const int R = a.G * a.Sq;
-  const int64_t total = (int64_t)a.B * a.Hkv * R;
-  const int64_t idx = (int64_t)blockIdx.x * (256 / TPR) + threadIdx.x / TPR;
-  const int c4 = threadIdx.x % TPR;
-  if (idx >= total) return;
-  const int r = (int)(idx % R);
-  const int64_t bh = idx / R;
+  const int ntile_r = (R + BM - 1) / BM;
+  const int lane = threadIdx.x & 63, r4 = threadIdx.x >> 6;
+  const int db = blockIdx.y % DB, wave = blockIdx.y / DB;
+  const int tile = blockIdx.x % ntile_r;
+  const int64_t bh = blockIdx.x / ntile_r;
   const int hk = (int)(bh % a.Hkv);
   const int b = (int)(bh / a.Hkv);
+  const int n = lane & 31, hh = lane >> 5;
+  const int r = tile * BM + wave * 32 + n;
+  if (r >= R) return;
   const int g = r / a.Sq, i = r - g * a.Sq, h = hk * a.G + g;
   const float c = a.scale * kLog2e;
-  const int64_t p0 = bh * sp.nsplit * R + r;
+  const int64_t item0 = bh * sp.nsplit * ntile_r + tile;
+  const float *mlp = sp.part_ml + 2 * (item0 * BM + wave * 32 + n);
+  const int64_t ml_step = 2 * (int64_t)ntile_r * BM;
+  // Loads go out eight splits at a time (indices past the end repeat the last split
+  // and get weight zero): a loop of dependent loads would pay the memory latency per split.
+  constexpr int CH = 8;
+  const part_t *pp = sp.part_o + item0 * (BM * D) + (int64_t)wave * (32 * D) + (db * 4 + r4) * 256 + 4 * lane;
+  const int64_t po_step = (int64_t)ntile_r * (BM * D);
   float mx = -INFINITY;
-  for (int s = 0; s < sp.nsplit; ++s) mx = fmaxf(mx, sp.part_ml[2 * (p0 + (int64_t)s * R)]);
+  for (int s0 = 0; s0 < sp.nsplit; s0 += CH) {
+    float mv[CH];
+#pragma unroll
+    for (int j = 0; j < CH; ++j) mv[j] = mlp[min(s0 + j, sp.nsplit - 1) * ml_step];
+#pragma unroll
+    for (int j = 0; j < CH; ++j) mx = fmaxf(mx, mv[j]);
+  }
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   float lsum = 0.f;
-  if (mx != -INFINITY) {
-    for (int s = 0; s < sp.nsplit; ++s) {
-      const int64_t pr = p0 + (int64_t)s * R;
-      const f32x2 ml = *reinterpret_cast<const f32x2 *>(sp.part_ml + 2 * pr);
-      if (ml[0] == -INFINITY) continue;
-      const float w = fast_exp2((ml[0] - mx) * c);
-      lsum += w * ml[1];
-      const f32x4 po = *reinterpret_cast<const f32x4 *>(sp.part_o + pr * D + 4 * c4);
+  const float mref = mx == -INFINITY ? 0.f : mx;
+  for (int s0 = 0; s0 < sp.nsplit; s0 += CH) {
+    f32x2 ml[CH];
+    part4_t po[CH];
 #pragma unroll
-      for (int x = 0; x < 4; ++x) acc[x] += w * po[x];
+    for (int j = 0; j < CH; ++j) {
+      const int sj = min(s0 + j, sp.nsplit - 1);
+      ml[j] = *reinterpret_cast<const f32x2 *>(mlp + sj * ml_step);
+      po[j] = *reinterpret_cast<const part4_t *>(pp + sj * po_step);
+    }
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      // a split without a visible key has max -inf and sum 0: weight 0, not NaN
+      const bool live = s0 + j < sp.nsplit && ml[j][0] != -INFINITY;
+      const float e = live ? fast_exp2((ml[j][0] - mref) * c) : 0.f;
+      const float w = kPartNormalized ? e * ml[j][1] : e;
+      lsum += e * ml[j][1];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) acc[x] += live ? w * (float)po[j][x] : 0.f;
     }
   }
   const bool has = lsum > 0.f;
@@ -327,21 +388,21 @@ __global__ __launch_bounds__(256) void fwd_combine_kernel(const FwdArgs a, const
 #pragma unroll
   for (int x = 0; x < 4; ++x) w[x] = (bf16_t)(acc[x] * inv);
   bf16_t *optr = reinterpret_cast<bf16_t *>(a.o) + b * a.o_sb + (int64_t)i * a.o_ss + h * a.o_sh;
-  *reinterpret_cast<bf16x4 *>(optr + 4 * c4) = w;
-  if (a.lse != nullptr && c4 == 0)
+  *reinterpret_cast<bf16x4 *>(optr + 32 * db + 8 * r4 + 4 * hh) = w;
+  if (a.lse != nullptr && db == 0 && r4 == 0 && hh == 0)
     a.lse[((int64_t)b * a.H + h) * a.Sq + i] = has ? mx * a.scale + __logf(lsum) : 0.f;
 }
 
 template <int D, int NW, bool SPLIT>
 static int launch_fwd_t(const FwdArgs &a, const SplitArgs &sp, hipStream_t st) {
-  if (hipFuncSetAttribute(reinterpret_cast<const void *>(&fwd_bf16_kernel<D, NW, SPLIT>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)fwd_smem_bytes<D>()) != hipSuccess)
+  constexpr size_t smem = fwd_smem_bytes<D, SPLIT>();
+  if (!allow_dynamic_lds<&fwd_bf16_kernel<D, NW, SPLIT>>((int)smem))
     return BCATTN_ERR_LAUNCH;
   const int R = a.G * a.Sq;
   const int ntile_r = (R + 32 * NW - 1) / (32 * NW);
   hipLaunchKernelGGL((fwd_bf16_kernel<D, NW, SPLIT>),
                      dim3(xcd_grid((unsigned)(ntile_r * (SPLIT ? sp.nsplit : 1) * a.Hkv * a.B))), dim3(64 * NW),
-                     fwd_smem_bytes<D>(), st, a, sp);
+                     smem, st, a, sp);
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
 }
 
@@ -360,12 +421,12 @@ int launch_fwd_bf16(const FwdArgs &a, int D, hipStream_t st) {
   }
 }
 
-// How many ways to split the key axis so that about 1.5 workgroups per CU exist.
+// How many ways to split the key axis so that about one workgroup per CU exists.
 static void plan_split(int B, int Sq, int Sk0, int Sk, int H, int Hkv, int *nsplit, int *tps) {
   const int R = (H / Hkv) * Sq;
-  const int base = B * Hkv * ((R + 127) / 128);
+  const int base = B * Hkv * ((R + kSplitRows - 1) / kSplitRows);
   const int ntiles = (Sk0 + 63) / 64 + (Sk - Sk0 + 63) / 64;
-  int want = (384 + base - 1) / base;
+  int want = (kSplitTarget + base - 1) / base;
   if (want < 1) want = 1;
   if (want > ntiles) want = ntiles;
   *tps = (ntiles + want - 1) / want;
@@ -378,19 +439,19 @@ size_t kvcache_workspace_bytes(int B, int Sq, int Sk0, int Sk, int H, int Hkv, i
   *nsplit_out = ns;
   if (ns <= 1) return 0;
   const size_t R = (size_t)(H / Hkv) * Sq;
-  const size_t rows = (size_t)B * Hkv * ns * R;
-  return ((rows * (D + 2) * sizeof(float)) + 255) & ~(size_t)255;
+  const size_t rows = (size_t)B * Hkv * ns * ((R + kSplitRows - 1) / kSplitRows) * kSplitRows;
+  return split_ml_bytes(rows) + ((rows * D * sizeof(part_t) + 255) & ~(size_t)255);
 }
 
 template <int D>
 static int launch_split(const FwdArgs &a, const SplitArgs &sp, hipStream_t st) {
   const int R = a.G * a.Sq;
-  const int rc = launch_fwd_t<D, 4, true>(a, sp, st);
+  constexpr int NW = kSplitRows / 32;
+  const int rc = launch_fwd_t<D, NW, true>(a, sp, st);
   if (rc) return rc;
-  constexpr int RPB = 256 / (D / 4);
-  const int64_t rows = (int64_t)a.B * a.Hkv * R;
-  hipLaunchKernelGGL(fwd_combine_kernel<D>, dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, a,
-                     sp);
+  const int ntile_r = (R + kSplitRows - 1) / kSplitRows;
+  hipLaunchKernelGGL((fwd_combine_kernel<D, NW>), dim3((unsigned)(a.B * a.Hkv * ntile_r), NW * (D / 32)),
+                     dim3(256), 0, st, a, sp);
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
 }
 

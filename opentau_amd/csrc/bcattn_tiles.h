@@ -238,4 +238,48 @@ __device__ __forceinline__ void tile_pipeline(int first, int end, Next next, Iss
   }
 }
 
+// Short tile ranges (a split of the key axis): the tiles [first, end) are taken in
+// order, none is skipped, and as many as there are LDS stages are requested at once,
+// so that a range of at most NS tiles pays the memory latency once.  The caller has
+// already requested the first min(NS, end - first) tiles into stages 0.. (it can do
+// that before it knows anything else); tile_burst() requests the rest as stages
+// free up.   issue(t, StageC) / compute(StageC, t) as for tile_pipeline.
+template <int K, int LPT>
+__device__ __forceinline__ void wait_async_tiles_but(int newer) {
+  // wait until at most `newer` (0..K) whole tiles of this wave's loads are in flight
+  if constexpr (K == 0) {
+    wait_async_loads_but<0>();
+  } else {
+    if (newer >= K)
+      wait_async_loads_but<K * LPT>();
+    else
+      wait_async_tiles_but<K - 1, LPT>(newer);
+  }
+}
+template <int NS, int LPT, class Issue, class Compute>
+__device__ __forceinline__ void tile_burst(int first, int end, Issue issue, Compute compute) {
+  static_assert(NS >= 2 && NS * LPT <= 63 + LPT, "wait counts are 6-bit immediates");
+  int t = first;
+  auto step = [&](auto sc) {
+    constexpr int S = decltype(sc)::value;
+    // tiles requested after t so far: up to first+NS-1 at the start, t+NS-2 later
+    const int last_req = min(end - 1, t == first ? first + NS - 1 : t + NS - 2);
+    wait_async_tiles_but<NS - 1, LPT>(last_req - t);
+    tile_barrier();  // tile t is in LDS for every wave, and every wave is done with tile t-1
+    if (t > first && t - 1 + NS < end) issue(t - 1 + NS, StageC<(S + NS - 1) % NS>{});
+    compute(sc, t);
+    return ++t >= end;
+  };
+  if (t >= end) return;
+  for (;;) {
+    if (step(StageC<0>{})) break;
+    if (step(StageC<1>{})) break;
+    if constexpr (NS >= 3)
+      if (step(StageC<2>{})) break;
+    if constexpr (NS >= 4)
+      if (step(StageC<3>{})) break;
+    static_assert(NS <= 4, "at most four stages");
+  }
+}
+
 }  // namespace bcattn
