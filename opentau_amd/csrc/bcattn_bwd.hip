@@ -120,6 +120,10 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
     red_s[wave] = qmax_w;
     red_s[NW + wave] = any_w;
   }
+  const int nt_all = (a.Sk + 63) / 64;
+  const tile_summary_t *ksum = a.ksum + (int64_t)b * nt_all;
+  SummaryTable ktab;
+  ktab.fill(ksum, reinterpret_cast<tile_summary_t *>(smem + NS * STAGE), nt_all, tid, NT);
   __syncthreads();
   int qmax_g = kIntMin, any_g = 0;
 #pragma unroll
@@ -127,11 +131,12 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
     qmax_g = max(qmax_g, red_s[x]);
     any_g |= red_s[NW + x];
   }
+  // (values read from LDS count as per-lane; these are the same in every lane)
+  qmax_g = __builtin_amdgcn_readfirstlane(qmax_g);
+  any_g = __builtin_amdgcn_readfirstlane(any_g);
 
   const int Sk = a.Sk;
-  const int nt_all = (Sk + 63) / 64;
   const int nt = any_g ? nt_all : 0;
-  const tile_summary_t *ksum = a.ksum + (int64_t)b * nt_all;
 
   const bf16_t *kbase = reinterpret_cast<const bf16_t *>(a.k.ptr) + b * a.k.sb + hk * a.k.sh;
   const bf16_t *vbase = reinterpret_cast<const bf16_t *>(a.v.ptr) + b * a.v.sb + hk * a.v.sh;
@@ -144,21 +149,14 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   vld.init(tid, a.v.ss);
   const uint32_t kstep = (uint32_t)(64 * a.k.ss * 2), vstep = (uint32_t)(64 * a.v.ss * 2);
 
-  const_summary_t *ksum_s = scalar_view(ksum);
-  // First tile at or after t that some row of the workgroup can see, with its summary.
-  auto next_needed = [&](int t, tile_summary_t &sm) {
-    while (t < nt) {
-      sm = ksum_s[t];
-      if (sm.x <= qmax_g) break;
-      ++t;
-    }
-    return t;
-  };
-  auto issue = [&](int t, auto stage_c) {
-    const char *st = smem + decltype(stage_c)::value * STAGE;
-    kld.issue(krs, st, (uint32_t)t * kstep, wave);
-    vld.issue(vrs, st + T::kBytes, (uint32_t)t * vstep, wave);
-    load_row64_dwords(idrs, st + 2 * T::kBytes, (uint32_t)t * 256, lane);  // every wave, same data
+  // A tile is needed if some row of the workgroup can see one of its keys.
+  auto needed = [&](int t) { return ktab.at(t).x <= qmax_g; };
+  const uint32_t smem0 = lds_addr(smem);
+  auto issue = [&](int t, auto stage_c, auto, bool live) {
+    const uint32_t st = smem0 + decltype(stage_c)::value * STAGE;
+    kld.issue(rsrc_if(krs, live), st, (uint32_t)t * kstep, wave);
+    vld.issue(rsrc_if(vrs, live), st + T::kBytes, (uint32_t)t * vstep, wave);
+    load_row64_dwords(rsrc_if(idrs, live), st + 2 * T::kBytes, (uint32_t)t * 256, lane);  // every wave, same data
   };
   constexpr int LPT = 2 * TileLoad<D, NT>::kLoads + 1;  // loads per tile and wave
 
@@ -174,11 +172,10 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
     for (int x = 0; x < 16; ++x) dq[db][x] = 0.f;
   const float c = a.scale * kLog2e;
 
-  auto compute = [&](auto stage_c, const tile_summary_t sm) {
-    if (sm.x > qmax_w) return;  // wave-uniform: no row of this wave sees a key of the tile
-#ifdef IGLP
-    __builtin_amdgcn_iglp_opt(IGLP);
-#endif
+  auto compute = [&](auto stage_c, int t, auto bg) {
+    const tile_summary_t sm = ktab.at(t);
+    if (sm.x > qmax_w) return false;
+    bg(StageC<0>{});  // wave-uniform: no row of this wave sees a key of the tile
     const char *st = smem + decltype(stage_c)::value * STAGE;
     const char *Kt = st, *Vt = st + T::kBytes;
     const int *kb_s = reinterpret_cast<const int *>(st + 2 * T::kBytes);
@@ -227,10 +224,12 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
         for (int db = 0; db < DB; ++db) dq[db] = mfma32(ka[db], dsb[half], dq[db]);
       }
     }
+    return true;
   };
 
   // Two LDS stages: while tile t is being used, tile t+1 streams into the other one.
-  tile_pipeline<NS, LPT>(0, nt, next_needed, issue, compute);
+  settle_loads();
+  tile_pipeline<NS, LPT, 1>(0, nt, needed, issue, compute);
 
   if (rowok) {
     bf16_t *optr = reinterpret_cast<bf16_t *>(a.dq) + b * a.dq_sb + (int64_t)i * a.dq_ss + h * a.dq_sh;
@@ -257,6 +256,14 @@ constexpr size_t dq_smem_bytes() {
 // launches that each recompute S; this is what fits the register file at
 // head_dim 256, and at 128 it lets two waves share a SIMD).
 constexpr int kModeBoth = 0, kModeDV = 1, kModeDK = 2;
+
+// Spreads `parts` things over `slots` >= parts places in order: the part that belongs at
+// slot s (part p sits at slot p*slots/parts), or -1.
+constexpr int part_at_slot(int s, int slots, int parts) {
+  for (int p = 0; p < parts; ++p)
+    if (p * slots / parts == s) return p;
+  return -1;
+}
 
 template <int D, int NW, int MODE>
 __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
@@ -305,13 +312,17 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   const int kmax_w = wave_max_i(kv ? kb : kIntMin);
   const int allk_w = wave_min_i(kv ? 1 : 0);
   if (lane == 0) red_s[wave] = kmin_w;
+  const int nqt = a.Sq_pad / 64;
+  const tile_summary_t *qsum = a.qsum + (int64_t)b * nqt;
+  SummaryTable qtab;
+  qtab.fill(qsum, reinterpret_cast<tile_summary_t *>(smem + NS * STAGE), nqt, tid, NT);
   __syncthreads();
   int kmin_g = kIntMax;
 #pragma unroll
   for (int x = 0; x < NW; ++x) kmin_g = min(kmin_g, red_s[x]);
+  // (values read from LDS count as per-lane; this one is the same in every lane)
+  kmin_g = __builtin_amdgcn_readfirstlane(kmin_g);
 
-  const int nqt = Sqp / 64;
-  const tile_summary_t *qsum = a.qsum + (int64_t)b * nqt;
   const int nit = (kmin_g == kIntMax) ? 0 : a.G * nqt;
 
   const bf16_t *qb0 = reinterpret_cast<const bf16_t *>(a.q.ptr) + b * a.q.sb + (int64_t)hk * a.G * a.q.sh;
@@ -320,42 +331,60 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   const uint32_t qbytes = (uint32_t)(((int64_t)(Sq - 1) * a.q.ss + D) * 2);
   const uint32_t gbytes = (uint32_t)(((int64_t)(Sq - 1) * a.d_o.ss + D) * 2);
   const int64_t stat0 = ((int64_t)b * a.H + (int64_t)hk * a.G) * Sqp;  // first row of (b, first head)
-  const buf_rsrc_t lrs = make_rsrc(a.lse2 + stat0, (uint32_t)(a.G * Sqp * 4));
-  const buf_rsrc_t drs = make_rsrc(a.delta + stat0, (uint32_t)(a.G * Sqp * 4));
-  const buf_rsrc_t irs = make_rsrc(a.qbm + (int64_t)b * Sqp, (uint32_t)(Sqp * 4));
+  // One statistics row of the tile per wave (lse, delta, query ids; further waves repeat
+  // one): each wave keeps only the descriptor of the row it fetches.
+  const int stat_kind = wave % 3;
+  const buf_rsrc_t strs = stat_kind == 1   ? make_rsrc(a.delta + stat0, (uint32_t)(a.G * Sqp * 4))
+                          : stat_kind == 2 ? make_rsrc(a.qbm + (int64_t)b * Sqp, (uint32_t)(Sqp * 4))
+                                           : make_rsrc(a.lse2 + stat0, (uint32_t)(a.G * Sqp * 4));
+  const uint32_t stat_dst = 2 * T::kBytes + 256 * stat_kind;
   TileLoad<D, NT> qld, gld;
   qld.init(tid, a.q.ss);
   gld.init(tid, a.d_o.ss);
   const uint32_t qstep = (uint32_t)(64 * a.q.ss * 2), gstep = (uint32_t)(64 * a.d_o.ss * 2);
 
-  const_summary_t *qsum_s = scalar_view(qsum);
-  // Iterations run over (query head of the group, query tile); first needed one at or after it.
-  auto next_needed = [&](int it, tile_summary_t &sm) {
-    while (it < nit) {
-      sm = qsum_s[it % nqt];
-      if (sm.w > 0 && sm.y >= kmin_g) break;
-      ++it;
+  // Iterations run over (query head of the group, query tile), head-major.  The pipeline
+  // asks about iterations in increasing order, so (head, tile) follow `it` by counting
+  // instead of by division.
+  int at_g = 0, at_base = 0;  // head of the iteration asked about last, and its first iteration
+  auto seek = [&](int it) {
+    int g = at_g, base = at_base;
+    while (it >= base + nqt) base += nqt, ++g;
+    at_g = __builtin_amdgcn_readfirstlane(g);
+    at_base = __builtin_amdgcn_readfirstlane(base);
+  };
+  auto needed = [&](int it) {
+    seek(it);
+    const tile_summary_t sm = qtab.at(it - at_base);
+    return sm.w > 0 && sm.y >= kmin_g;
+  };
+  const uint32_t smem0 = lds_addr(smem);
+  // A tile is requested one load at a time (part p of LPT): the Q loads, the dO loads,
+  // then the wave's statistics row.  Part 0 works out where the tile is.
+  constexpr int KL = TileLoad<D, NT>::kLoads;
+  constexpr int LPT = 2 * KL + 1;  // loads per tile and wave
+  int req_g = 0, req_qt = 0;
+  auto issue = [&](int it, auto stage_c, auto part_c, bool live) {
+    constexpr int P = decltype(part_c)::value;
+    const uint32_t st = smem0 + decltype(stage_c)::value * STAGE;
+    if constexpr (P == 0) {
+      // (the head asked about last is this tile's or a later one: count back)
+      int g = at_g, qt = it - at_base;
+      while (qt < 0) qt += nqt, --g;
+      req_g = __builtin_amdgcn_readfirstlane(g), req_qt = __builtin_amdgcn_readfirstlane(qt);
     }
-    return it;
+    // (descriptors are rebuilt where they are used: scalar registers are the scarce ones)
+    if constexpr (P < KL) {
+      qld.template issue_one<P>(make_rsrc(qb0 + (int64_t)req_g * a.q.sh, live ? qbytes : 0u), st,
+                                (uint32_t)req_qt * qstep, wave);
+    } else if constexpr (P < 2 * KL) {
+      gld.template issue_one<P - KL>(make_rsrc(gb0 + (int64_t)req_g * a.d_o.sh, live ? gbytes : 0u), st + T::kBytes,
+                                     (uint32_t)req_qt * gstep, wave);
+    } else {
+      const uint32_t row = stat_kind == 2 ? (uint32_t)(req_qt * 64) * 4 : (uint32_t)(req_g * Sqp + req_qt * 64) * 4;
+      load_row64_dwords(rsrc_if(strs, live), st + stat_dst, row, lane);
+    }
   };
-  auto issue = [&](int it, auto stage_c) {
-    const char *st = smem + decltype(stage_c)::value * STAGE;
-    const int g = it / nqt, qt = it - g * nqt;
-    const buf_rsrc_t qrs = make_rsrc(qb0 + (int64_t)g * a.q.sh, qbytes);
-    const buf_rsrc_t grs = make_rsrc(gb0 + (int64_t)g * a.d_o.sh, gbytes);
-    qld.issue(qrs, st, (uint32_t)qt * qstep, wave);
-    gld.issue(grs, st + T::kBytes, (uint32_t)qt * gstep, wave);
-    // one statistics row per wave (further waves repeat one)
-    const char *aux = st + 2 * T::kBytes;
-    const uint32_t srow = (uint32_t)(g * Sqp + qt * 64) * 4;
-    if (wave % 3 == 1)
-      load_row64_dwords(drs, aux + 256, srow, lane);
-    else if (wave % 3 == 2)
-      load_row64_dwords(irs, aux + 512, (uint32_t)(qt * 64) * 4, lane);
-    else
-      load_row64_dwords(lrs, aux, srow, lane);
-  };
-  constexpr int LPT = 2 * TileLoad<D, NT>::kLoads + 1;  // loads per tile and wave
 
   RowAddr<D> rowa;
   rowa.init(lane);
@@ -382,7 +411,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   // 0x008 matrix, 0x100 LDS read, 0x002 vector ALU); MASKED is a compile-time copy
   // of "some pair of this tile may be masked", so the common case carries no
   // compare/select at all.
-  auto compute_t = [&](auto stage_c, auto masked_c) {
+  auto compute_t = [&](auto stage_c, auto masked_c, auto bg) {
     constexpr bool MASKED = decltype(masked_c)::value != 0;
     const char *st = smem + decltype(stage_c)::value * STAGE;
     const char *Qt = st, *Gt = st + T::kBytes;
@@ -392,17 +421,22 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
     f32x16 s[2], dp[WANT_DK ? 2 : 1];
     bf16x8 pb[2][2], dsb[2][2];
 
-    auto phase_a = [&](int mb) {
+    // The loads of the tile due in this step go out one at a time between the products
+    // of the two A phases.
+    auto phase_a = [&](auto mb_c) {
+      constexpr int mb = decltype(mb_c)::value;
 #pragma unroll
       for (int x = 0; x < 16; ++x) {
         s[mb][x] = 0.f;
         if (WANT_DK) dp[mb][x] = 0.f;
       }
-#pragma unroll
-      for (int ks = 0; ks < DK; ++ks) {
+      static_for<DK>([&](auto ks_c) {
+        constexpr int ks = decltype(ks_c)::value;
+        constexpr int part = part_at_slot(mb * DK + ks, 2 * DK, LPT);
+        if constexpr (part >= 0) bg(StageC<part>{});
         s[mb] = mfma32(rowa.read(Qt, 32 * mb, ks), kf[ks], s[mb]);
         if (WANT_DK) dp[mb] = mfma32(rowa.read(Gt, 32 * mb, ks), vf[ks], dp[mb]);
-      }
+      });
     };
     auto softmax = [&](int mb) {
 #pragma unroll
@@ -443,7 +477,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
     constexpr int NC = 2 * DB * PER;                                  // products of one C phase
     constexpr int VA = (MASKED ? 9 : 7) * 16 / (NA < NC ? NA : NC) + 1;  // vector ALU instr. per product
 
-    phase_a(0);
+    phase_a(StageC<0>{});
     {
       constexpr int kAhead = NA < 6 ? NA : 6;
       __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
@@ -456,7 +490,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
     }
     __builtin_amdgcn_sched_barrier(0);
 
-    phase_a(1);
+    phase_a(StageC<1>{});
     softmax(0);
     {
       constexpr int kAhead = NA < 4 ? NA : 4;
@@ -497,15 +531,21 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-  auto compute = [&](auto stage_c, const tile_summary_t sm) {
-    if (sm.y < kmin_w) return;  // wave-uniform: no key of this wave is seen by the tile
+  auto compute = [&](auto stage_c, int it, auto bg) {
+    // (the head of iteration `it` is at most the one asked about last: count its tiles back)
+    int qt = it - at_base;
+    while (qt < 0) qt += nqt;
+    const tile_summary_t sm = qtab.at(__builtin_amdgcn_readfirstlane(qt));
+    if (sm.y < kmin_w) return false;  // wave-uniform: no key of this wave is seen by the tile
     if (sm.z != 0 && allk_w != 0 && kmax_w <= sm.x)
-      compute_t(stage_c, StageC<0>{});  // every pair of the tile attends
+      compute_t(stage_c, StageC<0>{}, bg);  // every pair of the tile attends
     else
-      compute_t(stage_c, StageC<1>{});
+      compute_t(stage_c, StageC<1>{}, bg);
+    return true;
   };
 
-  tile_pipeline<NS, LPT>(0, nit, next_needed, issue, compute);
+  settle_loads();
+  tile_pipeline<NS, LPT, LPT>(0, nit, needed, issue, compute);
 
   if (jok) {
     bf16_t *dkp = reinterpret_cast<bf16_t *>(a.dk) + b * a.dk_sb + (int64_t)j * a.dk_ss + hk * a.dk_sh;
@@ -533,11 +573,12 @@ constexpr size_t dkv_smem_bytes() {
 
 template <int D, int NW, int MODE>
 static int launch_dkv(const BwdArgs &a, hipStream_t st) {
-  if (!allow_dynamic_lds<&bwd_dkv_kernel<D, NW, MODE>>((int)dkv_smem_bytes<D>()))
-    return BCATTN_ERR_LAUNCH;
+  if (!allow_dynamic_lds<&bwd_dkv_kernel<D, NW, MODE>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
+  if (!summary_table_fits(dkv_smem_bytes<D>(), a.Sq_pad / 64)) return BCATTN_ERR_UNSUPPORTED;
+  const size_t smem = dkv_smem_bytes<D>() + (size_t)(a.Sq_pad / 64) * sizeof(tile_summary_t);
   const int nkt = (a.Sk + 32 * NW - 1) / (32 * NW);
   hipLaunchKernelGGL((bwd_dkv_kernel<D, NW, MODE>), dim3(xcd_grid((unsigned)(nkt * a.Hkv * a.B))),
-                     dim3(64 * NW), dkv_smem_bytes<D>(), st, a);
+                     dim3(64 * NW), smem, st, a);
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
 }
 
@@ -545,8 +586,8 @@ static int launch_dkv(const BwdArgs &a, hipStream_t st) {
 // runs as two launches (dV, then dK).
 template <int D, int NWQ, int NWK, bool SPLIT>
 static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
-  if (!allow_dynamic_lds<&bwd_dq_kernel<D, NWQ>>((int)dq_smem_bytes<D>()))
-    return BCATTN_ERR_LAUNCH;
+  if (!allow_dynamic_lds<&bwd_dq_kernel<D, NWQ>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
+  if (!summary_table_fits(dq_smem_bytes<D>(), (a.Sk + 63) / 64)) return BCATTN_ERR_UNSUPPORTED;
   if (a.stages & BCATTN_BWD_DELTA) {
     constexpr int RPB = 256 / (D / 8);
     const int64_t rows = (int64_t)a.B * a.H * a.Sq_pad;
@@ -555,8 +596,9 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
   if (a.stages & BCATTN_BWD_DQ) {
     const int R = a.G * a.Sq;
     const int ntile_r = (R + 32 * NWQ - 1) / (32 * NWQ);
+    const size_t smem = dq_smem_bytes<D>() + (size_t)((a.Sk + 63) / 64) * sizeof(tile_summary_t);
     hipLaunchKernelGGL((bwd_dq_kernel<D, NWQ>), dim3(xcd_grid((unsigned)(ntile_r * a.Hkv * a.B))), dim3(64 * NWQ),
-                       dq_smem_bytes<D>(), st, a);
+                       smem, st, a);
   }
   if (a.stages & BCATTN_BWD_DKV) {
     int rc;
@@ -575,11 +617,7 @@ int launch_bwd_bf16(const BwdArgs &a, int D, hipStream_t st) {
     case 64:
       return launch_bwd_d<64, 4, 4, false>(a, st);
     case 128:
-#ifdef DKV128_SPLIT
-      return R >= 1024 ? launch_bwd_d<128, 8, 8, true>(a, st) : launch_bwd_d<128, 4, 4, false>(a, st);
-#else
       return R >= 1024 ? launch_bwd_d<128, 8, 4, false>(a, st) : launch_bwd_d<128, 4, 4, false>(a, st);
-#endif
     case 256:
       return launch_bwd_d<256, 4, 4, true>(a, st);
     default:

@@ -234,6 +234,15 @@ inline bool allow_dynamic_lds(int bytes) {
   return true;
 }
 
+// The tile summaries a workgroup walks are copied to LDS after its tile stages; a
+// sequence with more tiles than fit in the CU's 160 KB is refused by the launcher
+// (more than 100 000 positions at head_dim 256, twice that at 128).
+constexpr size_t kLdsBytes = 160 * 1024;
+inline bool summary_table_fits(size_t stage_bytes, int tiles) {
+  const size_t room = kLdsBytes - 1024 - stage_bytes;  // 1 KB: the kernels' small static arrays
+  return (size_t)tiles * sizeof(tile_summary_t) <= room;
+}
+
 // kernel launchers, one translation unit each
 // Tile summaries and merged ids of a sequence given as two segments (n0 rows, then S - n0).
 int launch_summary(const int32_t *blk, const uint8_t *valid, int B, int n0, int S, int fill,

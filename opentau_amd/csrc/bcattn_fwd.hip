@@ -83,17 +83,19 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   k1ld.init(tid, a.k1.ss);
   v1ld.init(tid, a.v1.ss);
 
-  auto issue = [&](int t, auto stage_c) {
-    const char *st = smem + decltype(stage_c)::value * STAGE;
+  const uint32_t smem0 = lds_addr(smem);
+  auto issue_if = [&](int t, auto stage_c, bool live) {
+    const uint32_t st = smem0 + decltype(stage_c)::value * STAGE;
     if (t < nt0) {
-      k0ld.issue(k0rs, st, (uint32_t)(t * 64 * a.k0.ss * 2), wave);
-      v0ld.issue(v0rs, st + T::kBytes, (uint32_t)(t * 64 * a.v0.ss * 2), wave);
+      k0ld.issue(rsrc_if(k0rs, live), st, (uint32_t)(t * 64 * a.k0.ss * 2), wave);
+      v0ld.issue(rsrc_if(v0rs, live), st + T::kBytes, (uint32_t)(t * 64 * a.v0.ss * 2), wave);
     } else {
-      k1ld.issue(k1rs, st, (uint32_t)((t - nt0) * 64 * a.k1.ss * 2), wave);
-      v1ld.issue(v1rs, st + T::kBytes, (uint32_t)((t - nt0) * 64 * a.v1.ss * 2), wave);
+      k1ld.issue(rsrc_if(k1rs, live), st, (uint32_t)((t - nt0) * 64 * a.k1.ss * 2), wave);
+      v1ld.issue(rsrc_if(v1rs, live), st + T::kBytes, (uint32_t)((t - nt0) * 64 * a.v1.ss * 2), wave);
     }
-    load_row64_dwords(idrs, st + 2 * T::kBytes, (uint32_t)t * 256, lane);  // every wave, same data
+    load_row64_dwords(rsrc_if(idrs, live), st + 2 * T::kBytes, (uint32_t)t * 256, lane);  // every wave, same data
   };
+  auto issue = [&](int t, auto stage_c) { issue_if(t, stage_c, true); };
   constexpr int LPT = 2 * TileLoad<D, NT>::kLoads + 1;  // loads per tile and wave
 
   // A split workgroup has only a few tiles, so its start-up latency counts: its first
@@ -137,6 +139,8 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
     red_s[wave] = qmax_w;
     red_s[NW + wave] = any_w;
   }
+  SummaryTable ktab;
+  ktab.fill(ksum, reinterpret_cast<tile_summary_t *>(smem + NS * STAGE), SPLIT ? 0 : nt_all, tid, NT);
   __syncthreads();
   int qmax_g = kIntMin, any_g = 0;
 #pragma unroll
@@ -144,18 +148,14 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
     qmax_g = max(qmax_g, red_s[x]);
     any_g |= red_s[NW + x];
   }
+  // (values read from LDS count as per-lane; these are the same in every lane)
+  qmax_g = __builtin_amdgcn_readfirstlane(qmax_g);
+  any_g = __builtin_amdgcn_readfirstlane(any_g);
 
   const int nt = !any_g ? 0 : t_last;
   const_summary_t *ksum_s = scalar_view(ksum);
-  // First tile at or after t that some row of the workgroup can see, with its summary.
-  auto next_needed = [&](int t, tile_summary_t &sm) {
-    while (t < nt) {
-      sm = ksum_s[t];
-      if (sm.x <= qmax_g) break;
-      ++t;
-    }
-    return t;
-  };
+  // A tile is needed if some row of the workgroup can see one of its keys.
+  auto needed = [&](int t) { return ktab.at(t).x <= qmax_g; };
   RowAddr<D> rowa;
   rowa.init(lane);
   TrAddr<D> tra;
@@ -171,11 +171,8 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   float l = 0.f;        // this lane half's share of the running sum
   const float c = a.scale * kLog2e;
 
-  auto compute = [&](auto stage_c, const tile_summary_t sm) {
+  auto compute_sm = [&](auto stage_c, const tile_summary_t sm) {
     if (sm.x > qmax_w) return;  // wave-uniform: no row of this wave sees a key of the tile
-#ifdef IGLP
-    __builtin_amdgcn_iglp_opt(IGLP);
-#endif
     const char *st = smem + decltype(stage_c)::value * STAGE;
     const char *Kt = st, *Vt = st + T::kBytes;
     const int *kb_s = reinterpret_cast<const int *>(st + 2 * T::kBytes);
@@ -265,13 +262,21 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
     auto compute_t = [&](auto stage_c, int t) {
       const tile_summary_t sm = sm_next;
       sm_next = ksum_s[min(t + 1, nt_all - 1)];
-      compute(stage_c, sm);
+      compute_sm(stage_c, sm);
     };
+    settle_loads();
     tile_burst<NS, LPT>(t_first, nt, issue, compute_t);
     wait_async_loads_but<0>();  // the early requests, if no row of the workgroup is valid
   } else {
     // While tile t is being used, the next needed tile(s) stream into the other stage(s).
-    tile_pipeline<NS, LPT>(t_first, nt, next_needed, issue, compute);
+    auto issue_part = [&](int t, auto stage_c, auto, bool live) { issue_if(t, stage_c, live); };
+    auto compute = [&](auto stage_c, int t, auto bg) {
+      bg(StageC<0>{});
+      compute_sm(stage_c, ktab.at(t));
+      return true;
+    };
+    settle_loads();
+    tile_pipeline<NS, LPT, 1>(t_first, nt, needed, issue_part, compute);
   }
 
   // ---- epilogue ----------------------------------------------------------------
@@ -320,7 +325,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
 }
 
 template <int D, bool SPLIT>
-constexpr size_t fwd_smem_bytes() {
+constexpr size_t fwd_stage_bytes() {
   return (SPLIT ? SplitStages<D>::value : FwdStages<D>::value) * (2 * (size_t)Tile<D>::kBytes + 256);
 }
 
@@ -395,9 +400,11 @@ __global__ __launch_bounds__(256) void fwd_combine_kernel(const FwdArgs a, const
 
 template <int D, int NW, bool SPLIT>
 static int launch_fwd_t(const FwdArgs &a, const SplitArgs &sp, hipStream_t st) {
-  constexpr size_t smem = fwd_smem_bytes<D, SPLIT>();
-  if (!allow_dynamic_lds<&fwd_bf16_kernel<D, NW, SPLIT>>((int)smem))
-    return BCATTN_ERR_LAUNCH;
+  constexpr size_t stages = fwd_stage_bytes<D, SPLIT>();
+  if (!allow_dynamic_lds<&fwd_bf16_kernel<D, NW, SPLIT>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
+  const int tiles = SPLIT ? 0 : (a.Sk0 + 63) / 64 + (a.Sk - a.Sk0 + 63) / 64;
+  if (!summary_table_fits(stages, tiles)) return BCATTN_ERR_UNSUPPORTED;
+  const size_t smem = stages + (size_t)tiles * sizeof(tile_summary_t);
   const int R = a.G * a.Sq;
   const int ntile_r = (R + 32 * NW - 1) / (32 * NW);
   hipLaunchKernelGGL((fwd_bf16_kernel<D, NW, SPLIT>),

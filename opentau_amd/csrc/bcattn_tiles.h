@@ -50,28 +50,40 @@ __device__ __forceinline__ buf_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
   return r;
 }
 
-// Byte address of an LDS location, as the hardware counts it.
+// The same descriptor, or (live == false) one over zero bytes: loads through it fetch
+// nothing and deliver zeros.
+__device__ __forceinline__ buf_rsrc_t rsrc_if(buf_rsrc_t r, bool live) {
+  r[2] = live ? r[2] : 0;
+  return r;
+}
+
+// Byte address of an LDS location, as the hardware counts it (uniform: call it once on
+// the base of the dynamic LDS and add offsets to the result).
 __device__ __forceinline__ uint32_t lds_addr(const void *p) {
-  return (uint32_t)(uintptr_t)((__attribute__((address_space(3))) const char *)p);
+  return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)((__attribute__((address_space(3))) const char *)p));
 }
 
 // Asynchronous global -> LDS copy, 16 (or 4) bytes per lane: lane l reads
 // base + voff + soff and writes LDS byte lds_base + 16*l (4*l).  Issued as
-// assembly so that the compiler does not order later LDS reads of the *other*
-// stage behind it; completion is awaited explicitly with wait_async_loads().
+// assembly, and without a memory clobber, so that the compiler neither orders LDS
+// reads of the *other* stages behind it nor stops moving them across it; the
+// waits and barriers of the tile loop (which do clobber memory) are what orders
+// the copy against the reads of its own stage.
+template <int IMM>
 __device__ __forceinline__ void dma16(buf_rsrc_t rsrc, uint32_t lds_base, uint32_t voff, uint32_t soff) {
+  // LDS address lds_base + IMM; the constant goes into the instruction, not into a register
   asm volatile(
-      "s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+      "s_add_u32 m0, %0, %4\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
       :
-      : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
-      : "memory", "m0");
+      : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff), "n"(IMM)
+      : "m0", "scc");
 }
 __device__ __forceinline__ void dma4(buf_rsrc_t rsrc, uint32_t lds_base, uint32_t voff, uint32_t soff) {
   asm volatile(
       "s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
       :
       : "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff)
-      : "memory", "m0");
+      : "m0");
 }
 
 // Per-thread source offsets of an asynchronous tile load.  The tile's kSlots
@@ -93,19 +105,32 @@ struct TileLoad {
       voff[x] = (uint32_t)(row * row_stride_elems * 2 + L * 16);
     }
   }
-  // `tile` is the LDS tile base, `soff` the byte offset of the tile's first row.
-  __device__ __forceinline__ void issue(buf_rsrc_t rsrc, const char *tile, uint32_t soff, int wave) const {
-    const uint32_t base = __builtin_amdgcn_readfirstlane(lds_addr(tile) + 1024u * (uint32_t)wave);
+  // `tile` is the LDS byte address of the tile, `soff` the byte offset of its first row
+  // in the source.
+  __device__ __forceinline__ void issue(buf_rsrc_t rsrc, uint32_t tile, uint32_t soff, int wave) const {
+    const uint32_t base = __builtin_amdgcn_readfirstlane(tile + 1024u * (uint32_t)wave);
     const uint32_t so = __builtin_amdgcn_readfirstlane(soff);
-#pragma unroll
-    for (int x = 0; x < kLoads; ++x) dma16(rsrc, base + (uint32_t)(x * NT * 16), voff[x], so);
+    issue_from<0>(rsrc, base, so);
+  }
+  // Load X of the tile alone (the same arguments as issue()).
+  template <int X>
+  __device__ __forceinline__ void issue_one(buf_rsrc_t rsrc, uint32_t tile, uint32_t soff, int wave) const {
+    static_assert(X < kLoads, "load index");
+    dma16<X * NT * 16>(rsrc, __builtin_amdgcn_readfirstlane(tile + 1024u * (uint32_t)wave), voff[X],
+                       __builtin_amdgcn_readfirstlane(soff));
+  }
+  template <int X>
+  __device__ __forceinline__ void issue_from(buf_rsrc_t rsrc, uint32_t base, uint32_t so) const {
+    if constexpr (X < kLoads) {
+      dma16<X * NT * 16>(rsrc, base, voff[X], so);
+      issue_from<X + 1>(rsrc, base, so);
+    }
   }
 };
 
-// 64 consecutive dwords -> LDS, one per lane (a whole wave must call it).
-__device__ __forceinline__ void load_row64_dwords(buf_rsrc_t rsrc, const void *dst, uint32_t soff, int lane) {
-  dma4(rsrc, __builtin_amdgcn_readfirstlane(lds_addr(dst)), (uint32_t)lane * 4,
-       __builtin_amdgcn_readfirstlane(soff));
+// 64 consecutive dwords -> LDS byte address dst, one per lane (a whole wave must call it).
+__device__ __forceinline__ void load_row64_dwords(buf_rsrc_t rsrc, uint32_t dst, uint32_t soff, int lane) {
+  dma4(rsrc, __builtin_amdgcn_readfirstlane(dst), (uint32_t)lane * 4, __builtin_amdgcn_readfirstlane(soff));
 }
 
 __device__ __forceinline__ void wait_async_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
@@ -164,11 +189,22 @@ struct TrAddr {
   }
 };
 
+// f(StageC<0>{}), ..., f(StageC<N-1>{})
+template <int N, class F>
+__device__ __forceinline__ void static_for(F f);
+
 // Compile-time stage index, so that stage offsets fold into immediates.
 template <int S>
 struct StageC {
   static constexpr int value = S;
 };
+template <int N, class F>
+__device__ __forceinline__ void static_for(F f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(StageC<N - 1>{});
+  }
+}
 
 // Tile summaries are read with scalar loads (uniform address, memory that no
 // kernel writes while this one runs): they come back through the scalar cache
@@ -176,6 +212,27 @@ struct StageC {
 typedef const __attribute__((address_space(4))) tile_summary_t const_summary_t;
 __device__ __forceinline__ const_summary_t *scalar_view(const tile_summary_t *p) {
   return (const_summary_t *)reinterpret_cast<uintptr_t>(p);
+}
+
+// The summaries of a row of tiles, kept in LDS: a read costs an LDS access instead
+// of a trip to memory, and the main loop holds no ordinary memory load at all (one
+// would be waited for with a count that also drains the asynchronous tile loads).
+struct SummaryTable {
+  const tile_summary_t *lds;
+  // every thread of the workgroup calls this; a barrier must follow before at()
+  __device__ __forceinline__ void fill(const tile_summary_t *src, tile_summary_t *dst, int n, int tid, int nthreads) {
+    lds = dst;
+    for (int i = tid; i < n; i += nthreads) dst[i] = src[i];
+  }
+  __device__ __forceinline__ tile_summary_t at(int t) const { return uniform_summary(lds[t]); }
+};
+
+// Wait for every ordinary load issued so far, in a form the compiler takes note of.
+// A kernel calls this once before its tile loop: the compiler does not see the
+// asynchronous tile loads, and a register whose load it believes pending at the loop
+// entry would be waited for inside the loop with counts that drain the tile loads.
+__device__ __forceinline__ void settle_loads() {
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0), other counters untouched
 }
 
 // Wait until at most N of this wave's asynchronous loads are still in flight.
@@ -189,45 +246,73 @@ __device__ __forceinline__ void wait_async_loads_but() {
 __device__ __forceinline__ void tile_barrier() { asm volatile("s_barrier" ::: "memory"); }
 
 // Walk the needed tiles of [first, end) with NS LDS stages, i.e. NS-1 tiles of
-// asynchronous loads in flight while one is computed on.
-//   next(t, sm)        first needed tile >= t (or end) and its summary
-//   issue(t, StageC)   start the loads of tile t into that stage; every wave must
-//                      issue exactly LPT loads
-//   compute(StageC, sm)
+// prefetch:
+//   needed(t)            does some row of the workgroup use tile t (reads the
+//                        tile's summary from the LDS table)
+//   issue(t, StageC, StageC<part>, live)   requests part `part` of NPARTS of tile t
+//                        into that stage; over all parts every wave must issue
+//                        exactly LPT loads.  With live == false the same loads go
+//                        out against an empty buffer (they fetch nothing): every
+//                        step then issues the same number of loads, which keeps
+//                        the wait counts fixed and the issue free of branches
+//   compute(StageC, t, bg) -> bool   bg(StageC<part>{}) requests one part of the tile
+//                        that is due in this step; a compute() that returns true
+//                        has called it for every part (spread between its matrix
+//                        products, so that no wave sits waiting for the address
+//                        unit with nothing in flight), one that returns false for none
 // The loop is written out over the stages so that every LDS address inside
-// compute() is a lane offset plus a compile-time constant.
-template <int NS, int LPT, class Next, class Issue, class Compute>
-__device__ __forceinline__ void tile_pipeline(int first, int end, Next next, Issue issue, Compute compute) {
+// compute() is a lane offset plus a compile-time constant.  Only tile indices
+// are carried from step to step (scalar registers are scarce in these kernels);
+// the answer for the tile the next search starts at is fetched one step early.
+template <int NS, int LPT, int NPARTS, class Needed, class Issue, class Compute>
+__device__ __forceinline__ void tile_pipeline(int first, int end, Needed needed, Issue issue, Compute compute) {
   static_assert(NS == 2 || NS == 3, "two or three stages");
-  tile_summary_t s0 = {0, 0, 0, 0}, s1 = s0, s2 = s0;
-  int t0 = next(first, s0);
+  int ahead_t = -1;
+  bool ahead_ok = false;
+  // first needed tile at or after t (tile indices are uniform: keep them in scalar registers)
+  auto find = [&](int t) {
+    while (t < end) {
+      if (t == ahead_t ? ahead_ok : needed(t)) break;
+      ++t;
+    }
+    return __builtin_amdgcn_readfirstlane(t);
+  };
+  auto look_ahead = [&](int t) {
+    ahead_t = t;
+    if (t < end) ahead_ok = needed(t);
+  };
+  auto issue_all = [&](int t, auto sc, bool live) {
+    static_for<NPARTS>([&](auto part) { issue(t, sc, part, live); });
+  };
+  int t0 = find(first);
   if (t0 >= end) return;
-  issue(t0, StageC<0>{});
+  issue_all(t0, StageC<0>{}, true);
   int t1 = end, t2 = end;
   if (NS == 3) {
-    t1 = next(t0 + 1, s1);
-    if (t1 < end) issue(t1, StageC<1>{});
+    t1 = find(t0 + 1);
+    issue_all(t1 < end ? t1 : t0, StageC<1>{}, t1 < end);
   }
+  look_ahead((NS == 3 ? t1 : t0) + 1);
   auto step = [&](auto sc) {
     constexpr int S = decltype(sc)::value;
+    constexpr StageC<(S + NS - 1) % NS> into{};
     if (NS == 2) {
-      t1 = next(t0 + 1, s1);
+      t1 = find(t0 + 1);
       wait_async_loads_but<0>();
-      tile_barrier();
-      if (t1 < end) issue(t1, StageC<(S + 1) % 2>{});
-      compute(sc, s0);
-      t0 = t1, s0 = s1;
     } else {
-      t2 = t1 < end ? next(t1 + 1, s2) : end;
-      if (t1 < end)
-        wait_async_loads_but<LPT>();  // the newer tile may still be in flight
-      else
-        wait_async_loads_but<0>();
-      tile_barrier();
-      if (t2 < end) issue(t2, StageC<(S + 2) % 3>{});
-      compute(sc, s0);
-      t0 = t1, s0 = s1, t1 = t2, s1 = s2;
+      t2 = t1 < end ? find(t1 + 1) : end;
+      wait_async_loads_but<LPT>();  // the newer tile stays in flight
     }
+    tile_barrier();
+    const int tn = NS == 2 ? t1 : t2;  // the tile due in this step, if any
+    look_ahead(tn + 1);
+    const bool due = tn < end;
+    const int tq = due ? tn : t0;
+    if (!compute(sc, t0, [&](auto part) { issue(tq, into, part, due); })) issue_all(tq, into, due);
+    if (NS == 2)
+      t0 = t1;
+    else
+      t0 = t1, t1 = t2;
     return t0 >= end;
   };
   for (;;) {
@@ -236,6 +321,7 @@ __device__ __forceinline__ void tile_pipeline(int first, int end, Next next, Iss
     if (NS == 3)
       if (step(StageC<2>{})) break;
   }
+  wait_async_loads_but<0>();  // the empty requests of the last steps
 }
 
 // Short tile ranges (a split of the key axis): the tiles [first, end) are taken in
