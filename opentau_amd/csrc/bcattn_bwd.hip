@@ -69,8 +69,8 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   using T = Tile<D>;
   constexpr int NT = 64 * NW, BM = 32 * NW;
   constexpr int DK = D / 16, DB = D / 32;
-  constexpr int STAGE = 2 * T::kBytes + 256;  // K tile, V tile, 64 key ids
   constexpr int NS = BwdStages<D>::value;
+  using L = StageLayout<D, NS, 256>;  // per stage: K tile, V tile; 64 key ids
 
   extern __shared__ __align__(1024) char smem[];
   __shared__ int red_s[2 * NW];
@@ -78,6 +78,9 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
+#ifdef WAVE_PRIO
+  if (NW == 8 && wave >= 4) __builtin_amdgcn_s_setprio(WAVE_PRIO);
+#endif
 
   const int R = a.G * a.Sq;
   const int ntile_r = (R + BM - 1) / BM;
@@ -123,7 +126,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   const int nt_all = (a.Sk + 63) / 64;
   const tile_summary_t *ksum = a.ksum + (int64_t)b * nt_all;
   SummaryTable ktab;
-  ktab.fill(ksum, reinterpret_cast<tile_summary_t *>(smem + NS * STAGE), nt_all, tid, NT);
+  ktab.fill(ksum, reinterpret_cast<tile_summary_t *>(smem + L::kBytes), nt_all, tid, NT);
   __syncthreads();
   int qmax_g = kIntMin, any_g = 0;
 #pragma unroll
@@ -153,17 +156,17 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   auto needed = [&](int t) { return ktab.at(t).x <= qmax_g; };
   const uint32_t smem0 = lds_addr(smem);
   auto issue = [&](int t, auto stage_c, auto, bool live) {
-    const uint32_t st = smem0 + decltype(stage_c)::value * STAGE;
-    kld.issue(rsrc_if(krs, live), st, (uint32_t)t * kstep, wave);
-    vld.issue(rsrc_if(vrs, live), st + T::kBytes, (uint32_t)t * vstep, wave);
-    load_row64_dwords(rsrc_if(idrs, live), st + 2 * T::kBytes, (uint32_t)t * 256, lane);  // every wave, same data
+    constexpr int S = decltype(stage_c)::value;
+    kld.issue(rsrc_if(krs, live), smem0 + L::tile(S, 0), (uint32_t)t * kstep, wave);
+    vld.issue(rsrc_if(vrs, live), smem0 + L::tile(S, 1), (uint32_t)t * vstep, wave);
+    load_row64_dwords(rsrc_if(idrs, live), smem0 + L::aux(S), (uint32_t)t * 256, lane);  // every wave, same data
   };
   constexpr int LPT = 2 * TileLoad<D, NT>::kLoads + 1;  // loads per tile and wave
 
   RowAddr<D> rowa;
-  rowa.init(lane);
+  rowa.init(lane, smem0);
   TrAddr<D> tra;
-  tra.init(lane);
+  tra.init(lane, smem0);
 
   f32x16 dq[DB];
 #pragma unroll
@@ -176,9 +179,9 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
     const tile_summary_t sm = ktab.at(t);
     if (sm.x > qmax_w) return false;
     bg(StageC<0>{});  // wave-uniform: no row of this wave sees a key of the tile
-    const char *st = smem + decltype(stage_c)::value * STAGE;
-    const char *Kt = st, *Vt = st + T::kBytes;
-    const int *kb_s = reinterpret_cast<const int *>(st + 2 * T::kBytes);
+    constexpr int S = decltype(stage_c)::value;
+    constexpr int Kt = L::tile(S, 0), Vt = L::tile(S, 1);
+    const int *kb_s = reinterpret_cast<const int *>(smem + L::aux(S));
     const bool needmask = !(sm.z != 0 && sm.y <= qmin_w);
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb) {
@@ -191,8 +194,8 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
         bf16x8 fa[KB], fb[KB];
 #pragma unroll
         for (int ks = 0; ks < KB; ++ks) {
-          fa[ks] = rowa.read(Kt, 32 * mb, k0 + ks);
-          fb[ks] = rowa.read(Vt, 32 * mb, k0 + ks);
+          fa[ks] = rowa.template read<Kt>(32 * mb, k0 + ks);
+          fb[ks] = rowa.template read<Vt>(32 * mb, k0 + ks);
         }
 #pragma unroll
         for (int ks = 0; ks < KB; ++ks) {
@@ -219,7 +222,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
       for (int half = 0; half < 2; ++half) {
         bf16x8 ka[DB];
 #pragma unroll
-        for (int db = 0; db < DB; ++db) ka[db] = tra.read(Kt, 2 * mb + half, db);
+        for (int db = 0; db < DB; ++db) ka[db] = tra.template read<Kt>(2 * mb + half, db);
 #pragma unroll
         for (int db = 0; db < DB; ++db) dq[db] = mfma32(ka[db], dsb[half], dq[db]);
       }
@@ -247,7 +250,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
 
 template <int D>
 constexpr size_t dq_smem_bytes() {
-  return BwdStages<D>::value * (2 * (size_t)Tile<D>::kBytes + 256);
+  return StageLayout<D, BwdStages<D>::value, 256>::kBytes;
 }
 
 // ---- dK / dV ---------------------------------------------------------------------
@@ -271,8 +274,8 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   constexpr bool WANT_DV = MODE != kModeDK, WANT_DK = MODE != kModeDV;
   constexpr int NT = 64 * NW, BK = 32 * NW;
   constexpr int DK = D / 16, DB = D / 32;
-  constexpr int STAGE = 2 * T::kBytes + 3 * 256;  // Q tile, dO tile, lse2, delta, q ids
   constexpr int NS = BwdStages<D>::value;
+  using L = StageLayout<D, NS, 3 * 256>;  // per stage: Q tile, dO tile; lse2, delta, q ids
 
   extern __shared__ __align__(1024) char smem[];
   __shared__ int red_s[NW];
@@ -315,7 +318,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   const int nqt = a.Sq_pad / 64;
   const tile_summary_t *qsum = a.qsum + (int64_t)b * nqt;
   SummaryTable qtab;
-  qtab.fill(qsum, reinterpret_cast<tile_summary_t *>(smem + NS * STAGE), nqt, tid, NT);
+  qtab.fill(qsum, reinterpret_cast<tile_summary_t *>(smem + L::kBytes), nqt, tid, NT);
   __syncthreads();
   int kmin_g = kIntMax;
 #pragma unroll
@@ -337,7 +340,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   const buf_rsrc_t strs = stat_kind == 1   ? make_rsrc(a.delta + stat0, (uint32_t)(a.G * Sqp * 4))
                           : stat_kind == 2 ? make_rsrc(a.qbm + (int64_t)b * Sqp, (uint32_t)(Sqp * 4))
                                            : make_rsrc(a.lse2 + stat0, (uint32_t)(a.G * Sqp * 4));
-  const uint32_t stat_dst = 2 * T::kBytes + 256 * stat_kind;
+  const uint32_t stat_dst = 256 * stat_kind;
   TileLoad<D, NT> qld, gld;
   qld.init(tid, a.q.ss);
   gld.init(tid, a.d_o.ss);
@@ -366,7 +369,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   int req_g = 0, req_qt = 0;
   auto issue = [&](int it, auto stage_c, auto part_c, bool live) {
     constexpr int P = decltype(part_c)::value;
-    const uint32_t st = smem0 + decltype(stage_c)::value * STAGE;
+    constexpr int S = decltype(stage_c)::value;
     if constexpr (P == 0) {
       // (the head asked about last is this tile's or a later one: count back)
       int g = at_g, qt = it - at_base;
@@ -375,21 +378,22 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
     }
     // (descriptors are rebuilt where they are used: scalar registers are the scarce ones)
     if constexpr (P < KL) {
-      qld.template issue_one<P>(make_rsrc(qb0 + (int64_t)req_g * a.q.sh, live ? qbytes : 0u), st,
+      qld.template issue_one<P>(make_rsrc(qb0 + (int64_t)req_g * a.q.sh, live ? qbytes : 0u), smem0 + L::tile(S, 0),
                                 (uint32_t)req_qt * qstep, wave);
     } else if constexpr (P < 2 * KL) {
-      gld.template issue_one<P - KL>(make_rsrc(gb0 + (int64_t)req_g * a.d_o.sh, live ? gbytes : 0u), st + T::kBytes,
+      gld.template issue_one<P - KL>(make_rsrc(gb0 + (int64_t)req_g * a.d_o.sh, live ? gbytes : 0u),
+                                     smem0 + L::tile(S, 1),
                                      (uint32_t)req_qt * gstep, wave);
     } else {
       const uint32_t row = stat_kind == 2 ? (uint32_t)(req_qt * 64) * 4 : (uint32_t)(req_g * Sqp + req_qt * 64) * 4;
-      load_row64_dwords(rsrc_if(strs, live), st + stat_dst, row, lane);
+      load_row64_dwords(rsrc_if(strs, live), smem0 + L::aux(S) + stat_dst, row, lane);
     }
   };
 
   RowAddr<D> rowa;
-  rowa.init(lane);
+  rowa.init(lane, smem0);
   TrAddr<D> tra;
-  tra.init(lane);
+  tra.init(lane, smem0);
 
   f32x16 dk[WANT_DK ? DB : 1], dv[WANT_DV ? DB : 1];
 #pragma unroll
@@ -413,9 +417,9 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   // compare/select at all.
   auto compute_t = [&](auto stage_c, auto masked_c, auto bg) {
     constexpr bool MASKED = decltype(masked_c)::value != 0;
-    const char *st = smem + decltype(stage_c)::value * STAGE;
-    const char *Qt = st, *Gt = st + T::kBytes;
-    const float *lse_s = reinterpret_cast<const float *>(st + 2 * T::kBytes);
+    constexpr int S = decltype(stage_c)::value;
+    constexpr int Qt = L::tile(S, 0), Gt = L::tile(S, 1);
+    const float *lse_s = reinterpret_cast<const float *>(smem + L::aux(S));
     const float *delta_s = lse_s + 64;
     const int *qb_s = reinterpret_cast<const int *>(delta_s + 64);
     f32x16 s[2], dp[WANT_DK ? 2 : 1];
@@ -434,8 +438,8 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
         constexpr int ks = decltype(ks_c)::value;
         constexpr int part = part_at_slot(mb * DK + ks, 2 * DK, LPT);
         if constexpr (part >= 0) bg(StageC<part>{});
-        s[mb] = mfma32(rowa.read(Qt, 32 * mb, ks), kf[ks], s[mb]);
-        if (WANT_DK) dp[mb] = mfma32(rowa.read(Gt, 32 * mb, ks), vf[ks], dp[mb]);
+        s[mb] = mfma32(rowa.template read<Qt>(32 * mb, ks), kf[ks], s[mb]);
+        if (WANT_DK) dp[mb] = mfma32(rowa.template read<Gt>(32 * mb, ks), vf[ks], dp[mb]);
       });
     };
     auto softmax = [&](int mb) {
@@ -468,8 +472,8 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
       for (int half = 0; half < 2; ++half)
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-          if (WANT_DV) dv[db] = mfma32(tra.read(Gt, 2 * mb + half, db), pb[mb][half], dv[db]);
-          if (WANT_DK) dk[db] = mfma32(tra.read(Qt, 2 * mb + half, db), dsb[mb][half], dk[db]);
+          if (WANT_DV) dv[db] = mfma32(tra.template read<Gt>(2 * mb + half, db), pb[mb][half], dv[db]);
+          if (WANT_DK) dk[db] = mfma32(tra.template read<Qt>(2 * mb + half, db), dsb[mb][half], dk[db]);
         }
     };
     constexpr int PER = (WANT_DV ? 1 : 0) + (WANT_DK ? 1 : 0);
@@ -566,9 +570,434 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   }
 }
 
+// ---- dK / dV with paired waves --------------------------------------------------------
+// Two waves share 32 keys and split the work of a 32-query half tile in two equal parts:
+//   the P wave   holds the K fragments and the dV accumulators:
+//                S = Q K^T, P = exp2(c S - lse) (masked), leaves P as bf16 in an LDS
+//                exchange buffer, dV^T += dO^T P
+//   the dS wave  holds the V fragments and the dK accumulators:
+//                dP = dO V^T, takes P from the buffer, dS = P o (dP - delta), dK^T += Q^T dS
+// Each carries half the registers of the single-wave kernel, so two waves share a SIMD
+// and one's waits (LDS, vector ALU, tile requests, barriers) run in the shadow of the
+// other's matrix products.
+//
+// One barrier per half tile h orders the exchange:
+//   P wave,  between B(h-1) and B(h):  S(h), [softmax(h) beside dV(h-1)], P(h) -> X[h%2]
+//   dS wave, between B(h-1) and B(h):  dP(h), [X[(h-1)%2] -> dS(h-1) beside it], dK(h-1)
+// X[h%2] is written before B(h) and read after it, and is written again only after
+// B(h+1), which follows that read.  The tile of half h must be in LDS for every wave
+// before B(h-1) (S(h) starts right after it), so a wave waits for its own loads of
+// tile k+1 before B(2k+1); tile k+2 is requested after B(2k), when tile k-1, whose
+// stage it takes, was last used before B(2k).
+template <int D, int NP>
+__global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a) {
+  using T = Tile<D>;
+  constexpr int NW = 2 * NP, NT = 64 * NW, BK = 32 * NP;
+  constexpr int DK = D / 16, DB = D / 32;
+  constexpr int NS = 3;
+  using L = StageLayout<D, NS, 3 * 256>;  // per stage: Q tile, dO tile; lse2, delta, q ids
+  constexpr int XBYTES = NP * 2048;  // one exchange buffer: per pair the P of a half tile, bf16
+
+  extern __shared__ __align__(1024) char smem[];
+  __shared__ int red_s[NP];
+
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int n = lane & 31, hh = lane >> 5;
+  const bool pwave = wave < NP;  // wave-uniform role
+  const int pair = pwave ? wave : wave - NP;
+
+  const int Sk = a.Sk, Sq = a.Sq, Sqp = a.Sq_pad;
+  const int nkt = (Sk + BK - 1) / BK;
+  const int nitems = nkt * a.Hkv * a.B;
+  int bid = xcd_item(blockIdx.x, nitems);
+  if (bid >= nitems) return;
+  const int kt = __builtin_amdgcn_readfirstlane(bid % nkt);
+  bid /= nkt;
+  const int hk = __builtin_amdgcn_readfirstlane(bid % a.Hkv);
+  const int b = __builtin_amdgcn_readfirstlane(bid / a.Hkv);
+
+  // ---- this lane's key (the same in both waves of a pair) ----------------------------
+  const int j = kt * BK + pair * 32 + n;
+  const bool jok = j < Sk;
+  const int jj = jok ? j : Sk - 1;
+  const bool kv = jok && a.k_valid[(int64_t)b * Sk + jj] != 0;
+  const int kb = kv ? a.k_blk[(int64_t)b * Sk + jj] : kIntMax;
+  // K fragments in the P wave, V fragments in the dS wave
+  const bcattn::TensorArg &src = pwave ? a.k : a.v;
+  const bf16_t *fptr = reinterpret_cast<const bf16_t *>(src.ptr) + b * src.sb + (int64_t)jj * src.ss + hk * src.sh;
+  bf16x8 frag[DK];
+#pragma unroll
+  for (int ks = 0; ks < DK; ++ks) frag[ks] = *reinterpret_cast<const bf16x8 *>(fptr + 16 * ks + 8 * hh);
+  const int kmin_w = wave_min_i(kb);
+  const int kmax_w = wave_max_i(kv ? kb : kIntMin);
+  const int allk_w = wave_min_i(kv ? 1 : 0);
+  if (lane == 0 && pwave) red_s[pair] = kmin_w;
+  const int nqt = a.Sq_pad / 64;
+  const tile_summary_t *qsum = a.qsum + (int64_t)b * nqt;
+  SummaryTable qtab;
+  qtab.fill(qsum, reinterpret_cast<tile_summary_t *>(smem + L::kBytes + 2 * XBYTES), nqt, tid, NT);
+  __syncthreads();
+  int kmin_g = kIntMax;
+#pragma unroll
+  for (int x = 0; x < NP; ++x) kmin_g = min(kmin_g, red_s[x]);
+  kmin_g = __builtin_amdgcn_readfirstlane(kmin_g);  // read from LDS, but the same in every lane
+  const int nit = (kmin_g == kIntMax) ? 0 : a.G * nqt;
+
+  const bf16_t *qb0 = reinterpret_cast<const bf16_t *>(a.q.ptr) + b * a.q.sb + (int64_t)hk * a.G * a.q.sh;
+  const bf16_t *gb0 =
+      reinterpret_cast<const bf16_t *>(a.d_o.ptr) + b * a.d_o.sb + (int64_t)hk * a.G * a.d_o.sh;
+  const uint32_t qbytes = (uint32_t)(((int64_t)(Sq - 1) * a.q.ss + D) * 2);
+  const uint32_t gbytes = (uint32_t)(((int64_t)(Sq - 1) * a.d_o.ss + D) * 2);
+  const int64_t stat0 = ((int64_t)b * a.H + (int64_t)hk * a.G) * Sqp;
+  const int stat_kind = wave % 3;  // lse, delta, query ids: one row per wave, further waves repeat one
+  const buf_rsrc_t strs = stat_kind == 1   ? make_rsrc(a.delta + stat0, (uint32_t)(a.G * Sqp * 4))
+                          : stat_kind == 2 ? make_rsrc(a.qbm + (int64_t)b * Sqp, (uint32_t)(Sqp * 4))
+                                           : make_rsrc(a.lse2 + stat0, (uint32_t)(a.G * Sqp * 4));
+  const uint32_t stat_dst = 256 * stat_kind;
+  TileLoad<D, NT> qld, gld;
+  qld.init(tid, a.q.ss);
+  gld.init(tid, a.d_o.ss);
+  const uint32_t qstep = (uint32_t)(64 * a.q.ss * 2), gstep = (uint32_t)(64 * a.d_o.ss * 2);
+
+  // Iterations run over (query head of the group, query tile), head-major; (head, tile)
+  // follow the iteration index by counting.
+  int at_g = 0, at_base = 0;  // head of the iteration asked about last, and its first iteration
+  auto needed = [&](int it) {
+    int g = at_g, base = at_base;
+    while (it >= base + nqt) base += nqt, ++g;
+    at_g = __builtin_amdgcn_readfirstlane(g);
+    at_base = __builtin_amdgcn_readfirstlane(base);
+    const tile_summary_t sm = qtab.at(it - at_base);
+    return sm.w > 0 && sm.y >= kmin_g;
+  };
+  auto find = [&](int it) {
+    while (it < nit && !needed(it)) ++it;
+    return __builtin_amdgcn_readfirstlane(it);
+  };
+  // summary of an iteration at or before the one asked about last
+  auto summary_of = [&](int it) {
+    int qt = it - at_base;
+    while (qt < 0) qt += nqt;
+    return qtab.at(__builtin_amdgcn_readfirstlane(qt));
+  };
+  const uint32_t smem0 = lds_addr(smem);
+  constexpr int KL = TileLoad<D, NT>::kLoads;
+  constexpr int LPT = 2 * KL + 1;  // loads per tile and wave: Q, dO, one statistics row
+  int req_g = 0, req_qt = 0;
+  auto issue = [&](int it, auto stage_c, auto part_c, bool live) {
+    constexpr int P = decltype(part_c)::value;
+    constexpr int S = decltype(stage_c)::value;
+    if constexpr (P == 0) {
+      int g = at_g, qt = it - at_base;
+      while (qt < 0) qt += nqt, --g;
+      req_g = __builtin_amdgcn_readfirstlane(g), req_qt = __builtin_amdgcn_readfirstlane(qt);
+    }
+    if constexpr (P < KL) {
+      qld.template issue_one<P>(make_rsrc(qb0 + (int64_t)req_g * a.q.sh, live ? qbytes : 0u), smem0 + L::tile(S, 0),
+                                (uint32_t)req_qt * qstep, wave);
+    } else if constexpr (P < 2 * KL) {
+      gld.template issue_one<P - KL>(make_rsrc(gb0 + (int64_t)req_g * a.d_o.sh, live ? gbytes : 0u),
+                                     smem0 + L::tile(S, 1),
+                                     (uint32_t)req_qt * gstep, wave);
+    } else {
+      const uint32_t row = stat_kind == 2 ? (uint32_t)(req_qt * 64) * 4 : (uint32_t)(req_g * Sqp + req_qt * 64) * 4;
+      load_row64_dwords(rsrc_if(strs, live), smem0 + L::aux(S) + stat_dst, row, lane);
+    }
+  };
+  auto issue_all = [&](int it, auto stage_c, bool live) {
+    static_for<LPT>([&](auto part) { issue(it, stage_c, part, live); });
+  };
+
+  RowAddr<D> rowa;
+  rowa.init(lane, smem0);
+  TrAddr<D> tra;
+  tra.init(lane, smem0);
+  const float c = a.scale * kLog2e;
+  // this pair's part of an exchange buffer: the two 16-query halves of P, 1 KB each
+  char *xpair = smem + L::kBytes + pair * 2048 + lane * 16;
+
+  // The barrier of the exchange must find this wave's LDS writes done.
+  auto exchange_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+  f32x16 acc[DB];  // dV^T (P wave) or dK^T (dS wave)
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int x = 0; x < 16; ++x) acc[db][x] = 0.f;
+
+  // State carried from one half tile to the next: what the accumulating products of the
+  // previous half still need.
+  bf16x8 pend[2] = {};  // P wave: P(h-1) as bf16
+  f32x16 dp_prev = {};  // dS wave: dP(h-1)
+
+  // One half tile of the P wave: S(h) beside dV(h-1) (the chain of dependent products on
+  // one accumulator alternates with the independent ones on the dV blocks), then
+  // softmax(h) -> P(h), which goes to exchange buffer XCUR.  The dS wave does its vector
+  // ALU work first, so the two waves of a SIMD are out of phase.
+  // CUR / PREV: whether halves h and h-1 exist (first round: no h-1; last round: no h).
+  auto p_half = [&](auto cur_stage, auto mb_c, auto prev_stage, auto pmb_c, auto xcur_c, auto masked_c, auto cur_c,
+                    auto prev_c, auto bg) {
+    constexpr int mb = decltype(mb_c)::value, pmb = decltype(pmb_c)::value, xcur = decltype(xcur_c)::value;
+    constexpr bool MASKED = decltype(masked_c)::value != 0;
+    constexpr bool CUR = decltype(cur_c)::value != 0, PREV = decltype(prev_c)::value != 0;
+    constexpr int CS = decltype(cur_stage)::value, PS = decltype(prev_stage)::value;
+    constexpr int Qt = L::tile(CS, 0), Gp = L::tile(PS, 1);
+    f32x16 s;
+#pragma unroll
+    for (int x = 0; x < 16; ++x) s[x] = 0.f;
+    static_for<DK>([&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      constexpr int part = part_at_slot(i, DK, LPT);
+      if constexpr (part >= 0) bg(StageC<part>{});
+      if constexpr (CUR) s = mfma32(rowa.template read<Qt>(32 * mb, i), frag[i], s);
+      if constexpr (PREV)
+        acc[i % DB] = mfma32(tra.template read<Gp>(2 * pmb + i / DB, i % DB), pend[i / DB], acc[i % DB]);
+    });
+    {
+      constexpr int NR = (CUR ? DK : 0) + (PREV ? 2 * DK : 0);  // LDS reads of the products
+      constexpr int NM = (CUR ? DK : 0) + (PREV ? DK : 0);
+      constexpr int kAhead = 4;
+      __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+      for (int x = 0; x < NM; ++x) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, (NR - kAhead + NM - 1) / NM, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (CUR) {
+      const float *lse_s = reinterpret_cast<const float *>(smem + L::aux(CS));
+      const int *qb_s = reinterpret_cast<const int *>(lse_s + 128);
+      char *xb = xpair + xcur * XBYTES;
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        float p[8];
+#pragma unroll
+        for (int r2 = 0; r2 < 2; ++r2) {
+          const int r4 = 2 * half + r2;
+          const int q0 = 32 * mb + 8 * r4 + 4 * hh;
+          const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lse_s + q0);
+          i32x4 qb4 = {0, 0, 0, 0};
+          if (MASKED) qb4 = *reinterpret_cast<const i32x4 *>(qb_s + q0);
+#pragma unroll
+          for (int x = 0; x < 4; ++x) {
+            float pv = fast_exp2(s[4 * r4 + x] * c - lse4[x]);
+            if (MASKED && kb > qb4[x]) pv = 0.f;
+            p[4 * r2 + x] = pv;
+          }
+        }
+        pend[half] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
+        *reinterpret_cast<bf16x8 *>(xb + half * 1024) = pend[half];
+      }
+    }
+  };
+  // One half tile of the dS wave: P(h-1) from the other exchange buffer, dS(h-1) =
+  // P o (dP(h-1) - delta), then dK(h-1) beside dP(h).
+  auto ds_half = [&](auto cur_stage, auto mb_c, auto prev_stage, auto pmb_c, auto xcur_c, auto cur_c, auto prev_c,
+                     auto bg) {
+    constexpr int mb = decltype(mb_c)::value, pmb = decltype(pmb_c)::value, xcur = decltype(xcur_c)::value;
+    constexpr bool CUR = decltype(cur_c)::value != 0, PREV = decltype(prev_c)::value != 0;
+    constexpr int CS = decltype(cur_stage)::value, PS = decltype(prev_stage)::value;
+    constexpr int Gt = L::tile(CS, 1), Qp = L::tile(PS, 0);
+    bf16x8 dsb[2] = {};
+    if constexpr (PREV) {
+      const float *delta_s = reinterpret_cast<const float *>(smem + L::aux(PS)) + 64;
+      const char *xb = xpair + (1 - xcur) * XBYTES;
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const bf16x8 pb = *reinterpret_cast<const bf16x8 *>(xb + half * 1024);
+        float ds[8];
+#pragma unroll
+        for (int r2 = 0; r2 < 2; ++r2) {
+          const int r4 = 2 * half + r2;
+          const f32x4 del4 = *reinterpret_cast<const f32x4 *>(delta_s + 32 * pmb + 8 * r4 + 4 * hh);
+#pragma unroll
+          for (int x = 0; x < 4; ++x) ds[4 * r2 + x] = (float)pb[4 * r2 + x] * (dp_prev[4 * r4 + x] - del4[x]);
+        }
+        dsb[half] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    f32x16 dp;
+#pragma unroll
+    for (int x = 0; x < 16; ++x) dp[x] = 0.f;
+    static_for<DK>([&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      constexpr int part = part_at_slot(i, DK, LPT);
+      if constexpr (part >= 0) bg(StageC<part>{});
+      if constexpr (CUR) dp = mfma32(rowa.template read<Gt>(32 * mb, i), frag[i], dp);
+      if constexpr (PREV)
+        acc[i % DB] = mfma32(tra.template read<Qp>(2 * pmb + i / DB, i % DB), dsb[i / DB], acc[i % DB]);
+    });
+    {
+      constexpr int NR = (CUR ? DK : 0) + (PREV ? 2 * DK : 0);
+      constexpr int NM = (CUR ? DK : 0) + (PREV ? DK : 0);
+      constexpr int kAhead = 4;
+      __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+      for (int x = 0; x < NM; ++x) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, (NR - kAhead + NM - 1) / NM, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    dp_prev = dp;
+  };
+  // After the last half tile: its accumulating products alone.  The stage of the last
+  // tile is only known at run time here, which costs an address add per read but keeps
+  // this out of the unrolled loop (one copy, and no second set of accumulators).
+  auto p_last = [&](int stage) {
+    constexpr int A = L::tile(0, 1) / anchor_spacing<D>();
+    const int off = L::tile(0, 1) - A * anchor_spacing<D>() + stage * T::kBytes;
+#pragma unroll
+    for (int i = 0; i < DK; ++i)
+      acc[i % DB] = mfma32(tra.template read_from<A>(off + 16 * (2 + i / DB) * T::kRowBytes, i % DB), pend[i / DB],
+                           acc[i % DB]);
+  };
+  auto ds_last = [&](int stage) {
+    const float *delta_s = reinterpret_cast<const float *>(smem + L::aux(0) + stage * (3 * 256)) + 64;
+    const char *xb = xpair + XBYTES;  // the last half is an odd one
+    bf16x8 dsb[2];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const bf16x8 pb = *reinterpret_cast<const bf16x8 *>(xb + half * 1024);
+      float ds[8];
+#pragma unroll
+      for (int r2 = 0; r2 < 2; ++r2) {
+        const int r4 = 2 * half + r2;
+        const f32x4 del4 = *reinterpret_cast<const f32x4 *>(delta_s + 32 + 8 * r4 + 4 * hh);
+#pragma unroll
+        for (int x = 0; x < 4; ++x) ds[4 * r2 + x] = (float)pb[4 * r2 + x] * (dp_prev[4 * r4 + x] - del4[x]);
+      }
+      dsb[half] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
+    }
+    constexpr int A = L::tile(0, 0) / anchor_spacing<D>();
+    const int off = L::tile(0, 0) - A * anchor_spacing<D>() + stage * T::kBytes;
+#pragma unroll
+    for (int i = 0; i < DK; ++i)
+      acc[i % DB] = mfma32(tra.template read_from<A>(off + 16 * (2 + i / DB) * T::kRowBytes, i % DB), dsb[i / DB],
+                           acc[i % DB]);
+  };
+  auto no_bg = [](auto) {};
+  // The loop of one role.  Both roles run the same sequence of barriers.
+  auto run = [&](auto role_c) {
+    constexpr bool PW = decltype(role_c)::value == 0;
+    // Half h of iteration `it` (and the accumulating products of half h-1).
+    auto half_step = [&](auto cur_stage, int it, auto mb_c, auto prev_stage, auto pmb_c, auto xcur_c, auto cur_c,
+                         auto prev_c, auto bg) {
+      if constexpr (PW) {
+        bool masked = true;
+        if (decltype(cur_c)::value) {
+          const tile_summary_t sm = summary_of(it);
+          masked = !(sm.z != 0 && allk_w != 0 && kmax_w <= sm.x);
+        }
+        if (masked)
+          p_half(cur_stage, mb_c, prev_stage, pmb_c, xcur_c, StageC<1>{}, cur_c, prev_c, bg);
+        else  // every pair of the half attends
+          p_half(cur_stage, mb_c, prev_stage, pmb_c, xcur_c, StageC<0>{}, cur_c, prev_c, bg);
+      } else {
+        ds_half(cur_stage, mb_c, prev_stage, pmb_c, xcur_c, cur_c, prev_c, bg);
+      }
+    };
+    int t0 = find(0), last_stage = 0;
+    if (t0 >= nit) return;
+    issue_all(t0, StageC<0>{}, true);
+    int t1 = find(t0 + 1);
+    issue_all(t1 < nit ? t1 : t0, StageC<1>{}, t1 < nit);
+    wait_async_loads_but<LPT>();  // tile t0
+    exchange_barrier();
+    // very first tile: nothing to accumulate in its first half
+    {
+      const int t2 = t1 < nit ? find(t1 + 1) : nit;
+      half_step(StageC<0>{}, t0, StageC<0>{}, StageC<0>{}, StageC<1>{}, StageC<0>{}, StageC<1>{}, StageC<0>{}, no_bg);
+      exchange_barrier();  // B(0)
+      const bool due = t2 < nit;
+      const int tq = due ? t2 : t0;
+      half_step(StageC<0>{}, t0, StageC<1>{}, StageC<0>{}, StageC<0>{}, StageC<1>{}, StageC<1>{}, StageC<1>{},
+                [&](auto part) { issue(tq, StageC<2>{}, part, due); });
+      wait_async_loads_but<LPT>();  // tile t1
+      exchange_barrier();  // B(1)
+      t0 = t1, t1 = t2;
+    }
+    // tile t0 in stage S: halves 0 and 1; tile t1 (if any) must have landed before the
+    // second barrier; tile t2 is requested after the first, into the stage that the
+    // previous tile's last accumulating products (first half step) have then left
+    auto step = [&](auto sc) {
+      constexpr int S = decltype(sc)::value;
+      constexpr StageC<(S + NS - 1) % NS> before{};
+      constexpr StageC<(S + 2) % NS> into{};
+      if (t0 >= nit) {
+        last_stage = (S + NS - 1) % NS;
+        return true;
+      }
+      const int t2 = t1 < nit ? find(t1 + 1) : nit;
+      const bool due = t2 < nit;
+      const int tq = due ? t2 : t0;
+      // half 0 of this tile; the accumulating products of half 1 of the previous one
+      half_step(sc, t0, StageC<0>{}, before, StageC<1>{}, StageC<0>{}, StageC<1>{}, StageC<1>{}, no_bg);
+      exchange_barrier();  // B(2k): half 0's P is there; the previous tile's stage is free
+      half_step(sc, t0, StageC<1>{}, sc, StageC<0>{}, StageC<1>{}, StageC<1>{}, StageC<1>{},
+                [&](auto part) { issue(tq, into, part, due); });
+      wait_async_loads_but<LPT>();  // tile t1, for the S / dP of its first half
+      exchange_barrier();  // B(2k+1)
+      t0 = t1, t1 = t2;
+      return false;
+    };
+    for (;;) {
+      if (step(StageC<1>{})) break;
+      if (step(StageC<2>{})) break;
+      if (step(StageC<0>{})) break;
+    }
+    // one more round for the accumulating products of the last half
+    if constexpr (PW)
+      p_last(last_stage);
+    else
+      ds_last(last_stage);
+    wait_async_loads_but<0>();
+  };
+  settle_loads();
+  if (pwave)
+    run(StageC<0>{});
+  else
+    run(StageC<1>{});
+
+  if (jok) {
+    bf16_t *dst = pwave ? reinterpret_cast<bf16_t *>(a.dv) + b * a.dv_sb + (int64_t)j * a.dv_ss + hk * a.dv_sh
+                        : reinterpret_cast<bf16_t *>(a.dk) + b * a.dk_sb + (int64_t)j * a.dk_ss + hk * a.dk_sh;
+    const float mul = pwave ? 1.f : a.scale;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        bf16x4 w;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) w[x] = (bf16_t)(acc[db][4 * r4 + x] * mul);
+        *reinterpret_cast<bf16x4 *>(dst + 32 * db + 8 * r4 + 4 * hh) = w;
+      }
+  }
+}
+
+template <int D, int NP>
+constexpr size_t dkv_pair_smem_bytes() {
+  return StageLayout<D, 3, 3 * 256>::kBytes + 2 * (size_t)NP * 2048;
+}
+
+template <int D, int NP>
+static int launch_dkv_pair(const BwdArgs &a, hipStream_t st) {
+  if (!allow_dynamic_lds<&bwd_dkv_pair_kernel<D, NP>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
+  constexpr size_t fixed = dkv_pair_smem_bytes<D, NP>();
+  if (!summary_table_fits(fixed, a.Sq_pad / 64)) return BCATTN_ERR_UNSUPPORTED;
+  const size_t smem = fixed + (size_t)(a.Sq_pad / 64) * sizeof(tile_summary_t);
+  const int nkt = (a.Sk + 32 * NP - 1) / (32 * NP);
+  hipLaunchKernelGGL((bwd_dkv_pair_kernel<D, NP>), dim3(xcd_grid((unsigned)(nkt * a.Hkv * a.B))),
+                     dim3(128 * NP), smem, st, a);
+  return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
+}
+
 template <int D>
 constexpr size_t dkv_smem_bytes() {
-  return BwdStages<D>::value * (2 * (size_t)Tile<D>::kBytes + 3 * 256);
+  return StageLayout<D, BwdStages<D>::value, 3 * 256>::kBytes;
 }
 
 template <int D, int NW, int MODE>
@@ -584,7 +1013,7 @@ static int launch_dkv(const BwdArgs &a, hipStream_t st) {
 
 // NWQ: waves of the dQ kernel; NWK, SPLIT: waves of the dK/dV kernel and whether it
 // runs as two launches (dV, then dK).
-template <int D, int NWQ, int NWK, bool SPLIT>
+template <int D, int NWQ, int NWK, bool SPLIT, int PAIRS = 0>
 static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
   if (!allow_dynamic_lds<&bwd_dq_kernel<D, NWQ>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
   if (!summary_table_fits(dq_smem_bytes<D>(), (a.Sk + 63) / 64)) return BCATTN_ERR_UNSUPPORTED;
@@ -602,7 +1031,9 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
   }
   if (a.stages & BCATTN_BWD_DKV) {
     int rc;
-    if (SPLIT) {
+    if constexpr (PAIRS > 0) {
+      if ((rc = launch_dkv_pair<D, PAIRS>(a, st))) return rc;
+    } else if (SPLIT) {
       if ((rc = launch_dkv<D, NWK, kModeDV>(a, st)) || (rc = launch_dkv<D, NWK, kModeDK>(a, st))) return rc;
     } else if ((rc = launch_dkv<D, NWK, kModeBoth>(a, st))) {
       return rc;
@@ -617,7 +1048,7 @@ int launch_bwd_bf16(const BwdArgs &a, int D, hipStream_t st) {
     case 64:
       return launch_bwd_d<64, 4, 4, false>(a, st);
     case 128:
-      return R >= 1024 ? launch_bwd_d<128, 8, 4, false>(a, st) : launch_bwd_d<128, 4, 4, false>(a, st);
+      return R >= 1024 ? launch_bwd_d<128, 8, 4, false, 4>(a, st) : launch_bwd_d<128, 4, 4, false>(a, st);
     case 256:
       return launch_bwd_d<256, 4, 4, true>(a, st);
     default:

@@ -37,14 +37,17 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   constexpr int BM = 32 * NW;   // packed query rows per workgroup
   constexpr int DK = D / 16;    // contraction steps of K Q^T
   constexpr int DB = D / 32;    // 32-row blocks of O^T
-  constexpr int STAGE = 2 * T::kBytes + 256;  // K tile, V tile, 64 key ids
   constexpr int NS = SPLIT ? SplitStages<D>::value : FwdStages<D>::value;
+  using L = StageLayout<D, NS, 256>;  // per stage: K tile, V tile; 64 key ids
 
   extern __shared__ __align__(1024) char smem[];
   __shared__ int red_s[2 * NW];
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
+#ifdef WAVE_PRIO
+  if (NW == 8 && wave >= 4) __builtin_amdgcn_s_setprio(WAVE_PRIO);
+#endif
 
   const int R = a.G * a.Sq;
   const int ntile_r = (R + BM - 1) / BM;
@@ -85,15 +88,16 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
 
   const uint32_t smem0 = lds_addr(smem);
   auto issue_if = [&](int t, auto stage_c, bool live) {
-    const uint32_t st = smem0 + decltype(stage_c)::value * STAGE;
+    constexpr int S = decltype(stage_c)::value;
+    const uint32_t kt = smem0 + L::tile(S, 0), vt = smem0 + L::tile(S, 1);
     if (t < nt0) {
-      k0ld.issue(rsrc_if(k0rs, live), st, (uint32_t)(t * 64 * a.k0.ss * 2), wave);
-      v0ld.issue(rsrc_if(v0rs, live), st + T::kBytes, (uint32_t)(t * 64 * a.v0.ss * 2), wave);
+      k0ld.issue(rsrc_if(k0rs, live), kt, (uint32_t)(t * 64 * a.k0.ss * 2), wave);
+      v0ld.issue(rsrc_if(v0rs, live), vt, (uint32_t)(t * 64 * a.v0.ss * 2), wave);
     } else {
-      k1ld.issue(rsrc_if(k1rs, live), st, (uint32_t)((t - nt0) * 64 * a.k1.ss * 2), wave);
-      v1ld.issue(rsrc_if(v1rs, live), st + T::kBytes, (uint32_t)((t - nt0) * 64 * a.v1.ss * 2), wave);
+      k1ld.issue(rsrc_if(k1rs, live), kt, (uint32_t)((t - nt0) * 64 * a.k1.ss * 2), wave);
+      v1ld.issue(rsrc_if(v1rs, live), vt, (uint32_t)((t - nt0) * 64 * a.v1.ss * 2), wave);
     }
-    load_row64_dwords(rsrc_if(idrs, live), st + 2 * T::kBytes, (uint32_t)t * 256, lane);  // every wave, same data
+    load_row64_dwords(rsrc_if(idrs, live), smem0 + L::aux(S), (uint32_t)t * 256, lane);  // every wave, same data
   };
   auto issue = [&](int t, auto stage_c) { issue_if(t, stage_c, true); };
   constexpr int LPT = 2 * TileLoad<D, NT>::kLoads + 1;  // loads per tile and wave
@@ -140,7 +144,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
     red_s[NW + wave] = any_w;
   }
   SummaryTable ktab;
-  ktab.fill(ksum, reinterpret_cast<tile_summary_t *>(smem + NS * STAGE), SPLIT ? 0 : nt_all, tid, NT);
+  ktab.fill(ksum, reinterpret_cast<tile_summary_t *>(smem + L::kBytes), SPLIT ? 0 : nt_all, tid, NT);
   __syncthreads();
   int qmax_g = kIntMin, any_g = 0;
 #pragma unroll
@@ -157,9 +161,9 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   // A tile is needed if some row of the workgroup can see one of its keys.
   auto needed = [&](int t) { return ktab.at(t).x <= qmax_g; };
   RowAddr<D> rowa;
-  rowa.init(lane);
+  rowa.init(lane, smem0);
   TrAddr<D> tra;
-  tra.init(lane);
+  tra.init(lane, smem0);
 
   // ---- running state ---------------------------------------------------------
   f32x16 o[DB];
@@ -173,9 +177,9 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
 
   auto compute_sm = [&](auto stage_c, const tile_summary_t sm) {
     if (sm.x > qmax_w) return;  // wave-uniform: no row of this wave sees a key of the tile
-    const char *st = smem + decltype(stage_c)::value * STAGE;
-    const char *Kt = st, *Vt = st + T::kBytes;
-    const int *kb_s = reinterpret_cast<const int *>(st + 2 * T::kBytes);
+    constexpr int S = decltype(stage_c)::value;
+    constexpr int Kt = L::tile(S, 0), Vt = L::tile(S, 1);
+    const int *kb_s = reinterpret_cast<const int *>(smem + L::aux(S));
     // Two independent accumulator chains (the two 32-key halves) are interleaved:
     // back-to-back products on one accumulator would each wait for the previous one.
     f32x16 s[2];
@@ -190,8 +194,8 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
         bf16x8 ka0[KB], ka1[KB];
 #pragma unroll
         for (int ks = 0; ks < KB; ++ks) {
-          ka0[ks] = rowa.read(Kt, 0, k0 + ks);
-          ka1[ks] = rowa.read(Kt, 32, k0 + ks);
+          ka0[ks] = rowa.template read<Kt>(0, k0 + ks);
+          ka1[ks] = rowa.template read<Kt>(32, k0 + ks);
         }
 #pragma unroll
         for (int ks = 0; ks < KB; ++ks) {
@@ -249,7 +253,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
       for (int d0 = 0; d0 < DB; d0 += DBB) {
         bf16x8 va[DBB];
 #pragma unroll
-        for (int db = 0; db < DBB; ++db) va[db] = tra.read(Vt, kk, d0 + db);
+        for (int db = 0; db < DBB; ++db) va[db] = tra.template read<Vt>(kk, d0 + db);
 #pragma unroll
         for (int db = 0; db < DBB; ++db) o[d0 + db] = mfma32(va[db], pb[kk], o[d0 + db]);
       }
@@ -326,7 +330,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
 
 template <int D, bool SPLIT>
 constexpr size_t fwd_stage_bytes() {
-  return (SPLIT ? SplitStages<D>::value : FwdStages<D>::value) * (2 * (size_t)Tile<D>::kBytes + 256);
+  return StageLayout<D, (SPLIT ? SplitStages<D>::value : FwdStages<D>::value), 256>::kBytes;
 }
 
 // Merge the per-split partials.  A thread owns the same (wave, head_dim block, register

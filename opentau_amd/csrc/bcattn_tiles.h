@@ -135,25 +135,63 @@ __device__ __forceinline__ void load_row64_dwords(buf_rsrc_t rsrc, uint32_t dst,
 
 __device__ __forceinline__ void wait_async_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
+// LDS layout of a tile loop: the 2*NS tiles first, one after the other and grouped by
+// kind (tile w of stage s at (w*NS + s) tile sizes: the reads of one kind of tile then
+// mostly share an anchor, see below), then NS auxiliary areas of AUX bytes (ids,
+// statistics).
+template <int D, int NS, int AUX>
+struct StageLayout {
+  static constexpr int kTileBytes = 2 * NS * Tile<D>::kBytes;
+  static constexpr int kBytes = kTileBytes + NS * AUX;
+  static constexpr int tile(int s, int w) { return (w * NS + s) * Tile<D>::kBytes; }
+  static constexpr int aux(int s) { return kTileBytes + s * AUX; }
+};
+
 // ---------------------------------------------------------------------------
 // Operand reads.  The swizzle makes a read address a per-lane XOR pattern rather
-// than base + constant, so each lane computes its offsets once, before the main
-// loop; in the loop an address is (precomputed lane offset) + (compile-time
-// tile / stage / block constant), which folds into the instruction's immediate.
+// than base + constant, so each lane computes its addresses once, before the main
+// loop; in the loop an address is (precomputed lane address) + (compile-time tile /
+// row-block constant), and the constant must fit the 16-bit immediate of an LDS
+// instruction.  The tiles span more than 64 KB, so the lane addresses exist once
+// per "anchor" (every 48 KB, 64 KB at head_dim 256): a tile at byte T0 is read as
+// anchor T0 / spacing plus an immediate below 64 KB.  The anchors are made opaque to
+// the compiler (one assembly add each, at set-up), or it would fold them back into
+// one base and re-add the large constants in front of every read.
 // ---------------------------------------------------------------------------
+template <int D>
+constexpr int anchor_spacing() {
+  return D == 256 ? 65536 : 49152;
+}
+constexpr int kMaxAnchors = 3;
+__device__ __forceinline__ int opaque_add(int x, int c) {
+  int r;
+  asm("v_add_u32 %0, %1, %2" : "=v"(r) : "s"(c), "v"(x));
+  return r;
+}
+typedef const __attribute__((address_space(3))) bf16x8 lds_bf16x8_t;
 
 // Row operand of a 32x32x16 product: row (rbase + lane%32), columns
 // 16*ks + 8*(lane/32) .. +7.  rbase must be a multiple of 16 rows.
 template <int D>
 struct RowAddr {
-  int a[D / 16];
-  __device__ __forceinline__ void init(int lane) {
+  int a[kMaxAnchors][D / 16];
+  // lds0: LDS byte address of the tile area
+  __device__ __forceinline__ void init(int lane, uint32_t lds0) {
     const int n = lane & 31, hh = lane >> 5;
 #pragma unroll
-    for (int ks = 0; ks < D / 16; ++ks) a[ks] = Tile<D>::off(n, 2 * ks + hh);
+    for (int ks = 0; ks < D / 16; ++ks) {
+      a[0][ks] = (int)lds0 + Tile<D>::off(n, 2 * ks + hh);
+#pragma unroll
+      for (int i = 1; i < kMaxAnchors; ++i) a[i][ks] = opaque_add(a[0][ks], i * anchor_spacing<D>());
+    }
   }
-  __device__ __forceinline__ bf16x8 read(const char *tile, int rbase, int ks) const {
-    return *reinterpret_cast<const bf16x8 *>(tile + rbase * Tile<D>::kRowBytes + a[ks]);
+  // T0: byte offset of the tile in the tile area
+  template <int T0>
+  __device__ __forceinline__ bf16x8 read(int rbase, int ks) const {
+    constexpr int A = T0 / anchor_spacing<D>();
+    static_assert(A < kMaxAnchors, "tile beyond the last anchor");
+    const int addr = a[A][ks] + (T0 - A * anchor_spacing<D>()) + rbase * Tile<D>::kRowBytes;
+    return *reinterpret_cast<lds_bf16x8_t *>(static_cast<uintptr_t>((uint32_t)addr));
   }
 };
 
@@ -167,22 +205,37 @@ struct RowAddr {
 // columns 32*db + 16*(group%2) + 4*(i%4) .. +3.
 template <int D>
 struct TrAddr {
-  int lo[D / 32], hi[D / 32];
-  __device__ __forceinline__ void init(int lane) {
+  int lo[kMaxAnchors][D / 32], hi[kMaxAnchors][D / 32];
+  __device__ __forceinline__ void init(int lane, uint32_t lds0) {
     const int i = lane & 15, grp = (lane >> 4) & 1, hh = lane >> 5;
     const int row = 4 * hh + (i >> 2);
     const int slot = 2 * grp + ((i & 3) >> 1);
     const int byte = 8 * (i & 1);
 #pragma unroll
     for (int db = 0; db < D / 32; ++db) {
-      lo[db] = Tile<D>::off(row, 4 * db + slot) + byte;
-      hi[db] = Tile<D>::off(row + 8, 4 * db + slot) + byte;
+      lo[0][db] = (int)lds0 + Tile<D>::off(row, 4 * db + slot) + byte;
+      hi[0][db] = (int)lds0 + Tile<D>::off(row + 8, 4 * db + slot) + byte;
+#pragma unroll
+      for (int x = 1; x < kMaxAnchors; ++x) {
+        lo[x][db] = opaque_add(lo[0][db], x * anchor_spacing<D>());
+        hi[x][db] = opaque_add(hi[0][db], x * anchor_spacing<D>());
+      }
     }
   }
-  __device__ __forceinline__ bf16x8 read(const char *tile, int kk, int db) const {
-    const char *base = tile + 16 * kk * Tile<D>::kRowBytes;
-    const s16x4 l = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t *)(base + lo[db]));
-    const s16x4 h = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t *)(base + hi[db]));
+  template <int T0>
+  __device__ __forceinline__ bf16x8 read(int kk, int db) const {
+    constexpr int A = T0 / anchor_spacing<D>();
+    static_assert(A < kMaxAnchors, "tile beyond the last anchor");
+    return read_from<A>((T0 - A * anchor_spacing<D>()) + 16 * kk * Tile<D>::kRowBytes, db);
+  }
+  // The same with a tile offset known only at run time (costs an add per read): `off`
+  // is in bytes from anchor A.
+  template <int A>
+  __device__ __forceinline__ bf16x8 read_from(int off, int db) const {
+    const s16x4 l =
+        __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t *)static_cast<uintptr_t>((uint32_t)(lo[A][db] + off)));
+    const s16x4 h =
+        __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t *)static_cast<uintptr_t>((uint32_t)(hi[A][db] + off)));
     typedef short s16x8 __attribute__((ext_vector_type(8)));
     const s16x8 both = __builtin_shufflevector(l, h, 0, 1, 2, 3, 4, 5, 6, 7);
     return __builtin_bit_cast(bf16x8, both);
