@@ -655,6 +655,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
                           : stat_kind == 2 ? make_rsrc(a.qbm + (int64_t)b * Sqp, (uint32_t)(Sqp * 4))
                                            : make_rsrc(a.lse2 + stat0, (uint32_t)(a.G * Sqp * 4));
   const uint32_t stat_dst = 256 * stat_kind;
+  const int stat_gstride = stat_kind == 2 ? 0 : Sqp;  // the ids are per batch, the statistics per head
   TileLoad<D, NT> qld, gld;
   qld.init(tid, a.q.ss);
   gld.init(tid, a.d_o.ss);
@@ -684,15 +685,17 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   const uint32_t smem0 = lds_addr(smem);
   constexpr int KL = TileLoad<D, NT>::kLoads;
   constexpr int LPT = 2 * KL + 1;  // loads per tile and wave: Q, dO, one statistics row
+  // (head, tile) of the iteration to request: set by locate() before the parts go out,
+  // so that the parts themselves are free of branches
   int req_g = 0, req_qt = 0;
-  auto issue = [&](int it, auto stage_c, auto part_c, bool live) {
+  auto locate = [&](int it) {
+    int g = at_g, qt = it - at_base;  // the head asked about last is this one or a later one: count back
+    while (qt < 0) qt += nqt, --g;
+    req_g = __builtin_amdgcn_readfirstlane(g), req_qt = __builtin_amdgcn_readfirstlane(qt);
+  };
+  auto issue = [&](int, auto stage_c, auto part_c, bool live) {
     constexpr int P = decltype(part_c)::value;
     constexpr int S = decltype(stage_c)::value;
-    if constexpr (P == 0) {
-      int g = at_g, qt = it - at_base;
-      while (qt < 0) qt += nqt, --g;
-      req_g = __builtin_amdgcn_readfirstlane(g), req_qt = __builtin_amdgcn_readfirstlane(qt);
-    }
     if constexpr (P < KL) {
       qld.template issue_one<P>(make_rsrc(qb0 + (int64_t)req_g * a.q.sh, live ? qbytes : 0u), smem0 + L::tile(S, 0),
                                 (uint32_t)req_qt * qstep, wave);
@@ -701,11 +704,12 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
                                      smem0 + L::tile(S, 1),
                                      (uint32_t)req_qt * gstep, wave);
     } else {
-      const uint32_t row = stat_kind == 2 ? (uint32_t)(req_qt * 64) * 4 : (uint32_t)(req_g * Sqp + req_qt * 64) * 4;
+      const uint32_t row = (uint32_t)(req_g * stat_gstride + req_qt * 64) * 4;
       load_row64_dwords(rsrc_if(strs, live), smem0 + L::aux(S) + stat_dst, row, lane);
     }
   };
   auto issue_all = [&](int it, auto stage_c, bool live) {
+    locate(it);
     static_for<LPT>([&](auto part) { issue(it, stage_c, part, live); });
   };
 
@@ -731,11 +735,12 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   bf16x8 pend[2] = {};  // P wave: P(h-1) as bf16
   f32x16 dp_prev = {};  // dS wave: dP(h-1)
 
-  // One half tile of the P wave: S(h) beside dV(h-1) (the chain of dependent products on
-  // one accumulator alternates with the independent ones on the dV blocks), then
-  // softmax(h) -> P(h), which goes to exchange buffer XCUR.  The dS wave does its vector
-  // ALU work first, so the two waves of a SIMD are out of phase.
-  // CUR / PREV: whether halves h and h-1 exist (first round: no h-1; last round: no h).
+  // One half tile of the P wave: S(h) (a chain of dependent products), then softmax(h)
+  // -> P(h) beside the independent products of dV(h-1): the vector ALU work runs while
+  // the matrix unit works through products issued by this same wave.  P(h) goes to
+  // exchange buffer XCUR.  The dS wave has its vector ALU work in its first phase, so the
+  // two waves of a SIMD are out of phase as well.
+  // CUR / PREV: whether halves h and h-1 exist (the very first half has no h-1).
   auto p_half = [&](auto cur_stage, auto mb_c, auto prev_stage, auto pmb_c, auto xcur_c, auto masked_c, auto cur_c,
                     auto prev_c, auto bg) {
     constexpr int mb = decltype(mb_c)::value, pmb = decltype(pmb_c)::value, xcur = decltype(xcur_c)::value;
@@ -746,30 +751,35 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
     f32x16 s;
 #pragma unroll
     for (int x = 0; x < 16; ++x) s[x] = 0.f;
-    static_for<DK>([&](auto i_c) {
-      constexpr int i = decltype(i_c)::value;
-      constexpr int part = part_at_slot(i, DK, LPT);
-      if constexpr (part >= 0) bg(StageC<part>{});
-      if constexpr (CUR) s = mfma32(rowa.template read<Qt>(32 * mb, i), frag[i], s);
-      if constexpr (PREV)
-        acc[i % DB] = mfma32(tra.template read<Gp>(2 * pmb + i / DB, i % DB), pend[i / DB], acc[i % DB]);
-    });
-    {
-      constexpr int NR = (CUR ? DK : 0) + (PREV ? 2 * DK : 0);  // LDS reads of the products
-      constexpr int NM = (CUR ? DK : 0) + (PREV ? DK : 0);
-      constexpr int kAhead = 4;
+    if constexpr (CUR) {
+      static_for<DK>([&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        constexpr int part = part_at_slot(i, DK, LPT);
+        if constexpr (part >= 0) bg(StageC<part>{});
+        s = mfma32(rowa.template read<Qt>(32 * mb, i), frag[i], s);
+      });
+      constexpr int kAhead = DK < 6 ? DK : 6;
       __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
 #pragma unroll
-      for (int x = 0; x < NM; ++x) {
+      for (int x = 0; x < DK - kAhead; ++x) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, (NR - kAhead + NM - 1) / NM, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
       }
+      __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    } else {
+      static_for<LPT>([&](auto part) { bg(part); });
     }
-    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (PREV)
+      static_for<DK>([&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        acc[i % DB] = mfma32(tra.template read<Gp>(2 * pmb + i / DB, i % DB), pend[i / DB], acc[i % DB]);
+      });
     if constexpr (CUR) {
       const float *lse_s = reinterpret_cast<const float *>(smem + L::aux(CS));
       const int *qb_s = reinterpret_cast<const int *>(lse_s + 128);
       char *xb = xpair + xcur * XBYTES;
+      bf16x8 pnew[2];
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         float p[8];
@@ -787,13 +797,27 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
             p[4 * r2 + x] = pv;
           }
         }
-        pend[half] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
-        *reinterpret_cast<bf16x8 *>(xb + half * 1024) = pend[half];
+        pnew[half] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
+        *reinterpret_cast<bf16x8 *>(xb + half * 1024) = pnew[half];
+      }
+      pend[0] = pnew[0], pend[1] = pnew[1];
+    }
+    if constexpr (PREV) {
+      // per product of dV: its two transposed reads and a share of the softmax
+      constexpr int VA = CUR ? ((MASKED ? 9 : 7) * 16 + DK - 1) / DK : 0;
+      __builtin_amdgcn_sched_group_barrier(0x100, 4 + (CUR ? (MASKED ? 8 : 4) : 0), 0);
+#pragma unroll
+      for (int x = 0; x < DK; ++x) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        if (VA) __builtin_amdgcn_sched_group_barrier(0x002, VA, 0);
       }
     }
+    __builtin_amdgcn_sched_barrier(0);
   };
-  // One half tile of the dS wave: P(h-1) from the other exchange buffer, dS(h-1) =
-  // P o (dP(h-1) - delta), then dK(h-1) beside dP(h).
+  // One half tile of the dS wave: P(h-1) from the other exchange buffer and dS(h-1) =
+  // P o (dP(h-1) - delta) beside the products of dP(h) (which do not depend on it), then
+  // dK(h-1).
   auto ds_half = [&](auto cur_stage, auto mb_c, auto prev_stage, auto pmb_c, auto xcur_c, auto cur_c, auto prev_c,
                      auto bg) {
     constexpr int mb = decltype(mb_c)::value, pmb = decltype(pmb_c)::value, xcur = decltype(xcur_c)::value;
@@ -801,6 +825,18 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
     constexpr int CS = decltype(cur_stage)::value, PS = decltype(prev_stage)::value;
     constexpr int Gt = L::tile(CS, 1), Qp = L::tile(PS, 0);
     bf16x8 dsb[2] = {};
+    f32x16 dp;
+#pragma unroll
+    for (int x = 0; x < 16; ++x) dp[x] = 0.f;
+    if constexpr (CUR)
+      static_for<DK>([&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        constexpr int part = part_at_slot(i, DK, LPT);
+        if constexpr (part >= 0) bg(StageC<part>{});
+        dp = mfma32(rowa.template read<Gt>(32 * mb, i), frag[i], dp);
+      });
+    else
+      static_for<LPT>([&](auto part) { bg(part); });
     if constexpr (PREV) {
       const float *delta_s = reinterpret_cast<const float *>(smem + L::aux(PS)) + 64;
       const char *xb = xpair + (1 - xcur) * XBYTES;
@@ -818,30 +854,33 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
         dsb[half] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
       }
     }
-    __builtin_amdgcn_sched_barrier(0);
-    f32x16 dp;
+    if constexpr (CUR) {
+      // per product of dP: its row read and a share of the dS arithmetic
+      constexpr int VA = PREV ? (4 * 16 + DK - 1) / DK : 0;
+      __builtin_amdgcn_sched_group_barrier(0x100, (PREV ? 6 : 0) + 4, 0);
 #pragma unroll
-    for (int x = 0; x < 16; ++x) dp[x] = 0.f;
-    static_for<DK>([&](auto i_c) {
-      constexpr int i = decltype(i_c)::value;
-      constexpr int part = part_at_slot(i, DK, LPT);
-      if constexpr (part >= 0) bg(StageC<part>{});
-      if constexpr (CUR) dp = mfma32(rowa.template read<Gt>(32 * mb, i), frag[i], dp);
-      if constexpr (PREV)
-        acc[i % DB] = mfma32(tra.template read<Qp>(2 * pmb + i / DB, i % DB), dsb[i / DB], acc[i % DB]);
-    });
-    {
-      constexpr int NR = (CUR ? DK : 0) + (PREV ? 2 * DK : 0);
-      constexpr int NM = (CUR ? DK : 0) + (PREV ? DK : 0);
-      constexpr int kAhead = 4;
-      __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
-#pragma unroll
-      for (int x = 0; x < NM; ++x) {
+      for (int x = 0; x < DK; ++x) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, (NR - kAhead + NM - 1) / NM, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        if (VA) __builtin_amdgcn_sched_group_barrier(0x002, VA, 0);
       }
     }
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (PREV) {
+      static_for<DK>([&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        acc[i % DB] = mfma32(tra.template read<Qp>(2 * pmb + i / DB, i % DB), dsb[i / DB], acc[i % DB]);
+      });
+      constexpr int kAhead = DK < 4 ? DK : 4;
+      __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
+#pragma unroll
+      for (int x = 0; x < DK - kAhead; ++x) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
     dp_prev = dp;
   };
   // After the last half tile: its accumulating products alone.  The stage of the last
@@ -914,6 +953,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
       exchange_barrier();  // B(0)
       const bool due = t2 < nit;
       const int tq = due ? t2 : t0;
+      locate(tq);
       half_step(StageC<0>{}, t0, StageC<1>{}, StageC<0>{}, StageC<0>{}, StageC<1>{}, StageC<1>{}, StageC<1>{},
                 [&](auto part) { issue(tq, StageC<2>{}, part, due); });
       wait_async_loads_but<LPT>();  // tile t1
@@ -934,6 +974,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
       const int t2 = t1 < nit ? find(t1 + 1) : nit;
       const bool due = t2 < nit;
       const int tq = due ? t2 : t0;
+      locate(tq);
       // half 0 of this tile; the accumulating products of half 1 of the previous one
       half_step(sc, t0, StageC<0>{}, before, StageC<1>{}, StageC<0>{}, StageC<1>{}, StageC<1>{}, no_bg);
       exchange_barrier();  // B(2k): half 0's P is there; the previous tile's stage is free
