@@ -125,8 +125,6 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   }
   const int nt_all = (a.Sk + 63) / 64;
   const tile_summary_t *ksum = a.ksum + (int64_t)b * nt_all;
-  SummaryTable ktab;
-  ktab.fill(ksum, reinterpret_cast<tile_summary_t *>(smem + L::kBytes), nt_all, tid, NT);
   __syncthreads();
   int qmax_g = kIntMin, any_g = 0;
 #pragma unroll
@@ -153,7 +151,11 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   const uint32_t kstep = (uint32_t)(64 * a.k.ss * 2), vstep = (uint32_t)(64 * a.v.ss * 2);
 
   // A tile is needed if some row of the workgroup can see one of its keys.
-  auto needed = [&](int t) { return ktab.at(t).x <= qmax_g; };
+  NeededTable ktab;
+  ktab.fill(ksum, reinterpret_cast<i32x4 *>(smem + L::kBytes), nt_all, tid, NT,
+            [&](const tile_summary_t sm) { return sm.x <= qmax_g; });
+  __syncthreads();
+  auto find = [&](int t) { return ktab.at(t).x; };
   const uint32_t smem0 = lds_addr(smem);
   auto issue = [&](int t, auto stage_c, auto, bool live) {
     constexpr int S = decltype(stage_c)::value;
@@ -176,7 +178,8 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   const float c = a.scale * kLog2e;
 
   auto compute = [&](auto stage_c, int t, auto bg) {
-    const tile_summary_t sm = ktab.at(t);
+    const i32x4 e = ktab.at(t);
+    const tile_summary_t sm = {e.y, e.z, e.w, 0};
     if (sm.x > qmax_w) return false;
     bg(StageC<0>{});  // wave-uniform: no row of this wave sees a key of the tile
     constexpr int S = decltype(stage_c)::value;
@@ -232,7 +235,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
 
   // Two LDS stages: while tile t is being used, tile t+1 streams into the other one.
   settle_loads();
-  tile_pipeline<NS, LPT, 1>(0, nt, needed, issue, compute);
+  tile_pipeline<NS, LPT, 1>(0, nt, find, issue, compute);
 
   if (rowok) {
     bf16_t *optr = reinterpret_cast<bf16_t *>(a.dq) + b * a.dq_sb + (int64_t)i * a.dq_ss + h * a.dq_sh;
@@ -317,16 +320,21 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   if (lane == 0) red_s[wave] = kmin_w;
   const int nqt = a.Sq_pad / 64;
   const tile_summary_t *qsum = a.qsum + (int64_t)b * nqt;
-  SummaryTable qtab;
-  qtab.fill(qsum, reinterpret_cast<tile_summary_t *>(smem + L::kBytes), nqt, tid, NT);
   __syncthreads();
   int kmin_g = kIntMax;
 #pragma unroll
   for (int x = 0; x < NW; ++x) kmin_g = min(kmin_g, red_s[x]);
   // (values read from LDS count as per-lane; this one is the same in every lane)
   kmin_g = __builtin_amdgcn_readfirstlane(kmin_g);
+  // A query tile is needed if it has a valid query that sees some key of the workgroup.
+  NeededTable qtab;
+  qtab.fill(qsum, reinterpret_cast<i32x4 *>(smem + L::kBytes), nqt, tid, NT,
+            [&](const tile_summary_t sm) { return sm.w > 0 && sm.y >= kmin_g; });
+  __syncthreads();
 
-  const int nit = (kmin_g == kIntMax) ? 0 : a.G * nqt;
+  // Iterations run over (query head of the group, query tile), head-major; an iteration
+  // index is head << 16 | tile, so neither part needs a division.
+  const int nit = (kmin_g == kIntMax) ? 0 : a.G << 16;
 
   const bf16_t *qb0 = reinterpret_cast<const bf16_t *>(a.q.ptr) + b * a.q.sb + (int64_t)hk * a.G * a.q.sh;
   const bf16_t *gb0 =
@@ -346,20 +354,14 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   gld.init(tid, a.d_o.ss);
   const uint32_t qstep = (uint32_t)(64 * a.q.ss * 2), gstep = (uint32_t)(64 * a.d_o.ss * 2);
 
-  // Iterations run over (query head of the group, query tile), head-major.  The pipeline
-  // asks about iterations in increasing order, so (head, tile) follow `it` by counting
-  // instead of by division.
-  int at_g = 0, at_base = 0;  // head of the iteration asked about last, and its first iteration
-  auto seek = [&](int it) {
-    int g = at_g, base = at_base;
-    while (it >= base + nqt) base += nqt, ++g;
-    at_g = __builtin_amdgcn_readfirstlane(g);
-    at_base = __builtin_amdgcn_readfirstlane(base);
-  };
-  auto needed = [&](int it) {
-    seek(it);
-    const tile_summary_t sm = qtab.at(it - at_base);
-    return sm.w > 0 && sm.y >= kmin_g;
+  // first needed iteration at or after `it`: in its head, else the first of the next head
+  // (every head has the same needed tiles)
+  auto find = [&](int it) {
+    const int g = it >> 16, qt = it & 0xffff;
+    const int nn = qtab.at(qt < nqt ? qt : nqt).x;
+    if (nn < nqt) return (g << 16) | nn;
+    const int first = qtab.at(0).x;
+    return first < nqt ? ((g + 1) << 16) | first : nit;
   };
   const uint32_t smem0 = lds_addr(smem);
   // A tile is requested one load at a time (part p of LPT): the Q loads, the dO loads,
@@ -370,12 +372,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   auto issue = [&](int it, auto stage_c, auto part_c, bool live) {
     constexpr int P = decltype(part_c)::value;
     constexpr int S = decltype(stage_c)::value;
-    if constexpr (P == 0) {
-      // (the head asked about last is this tile's or a later one: count back)
-      int g = at_g, qt = it - at_base;
-      while (qt < 0) qt += nqt, --g;
-      req_g = __builtin_amdgcn_readfirstlane(g), req_qt = __builtin_amdgcn_readfirstlane(qt);
-    }
+    if constexpr (P == 0) req_g = it >> 16, req_qt = it & 0xffff;
     // (descriptors are rebuilt where they are used: scalar registers are the scarce ones)
     if constexpr (P < KL) {
       qld.template issue_one<P>(make_rsrc(qb0 + (int64_t)req_g * a.q.sh, live ? qbytes : 0u), smem0 + L::tile(S, 0),
@@ -536,10 +533,8 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
     __builtin_amdgcn_sched_barrier(0);
   };
   auto compute = [&](auto stage_c, int it, auto bg) {
-    // (the head of iteration `it` is at most the one asked about last: count its tiles back)
-    int qt = it - at_base;
-    while (qt < 0) qt += nqt;
-    const tile_summary_t sm = qtab.at(__builtin_amdgcn_readfirstlane(qt));
+    const i32x4 e = qtab.at(it & 0xffff);
+    const tile_summary_t sm = {e.y, e.z, e.w, 0};
     if (sm.y < kmin_w) return false;  // wave-uniform: no key of this wave is seen by the tile
     if (sm.z != 0 && allk_w != 0 && kmax_w <= sm.x)
       compute_t(stage_c, StageC<0>{}, bg);  // every pair of the tile attends
@@ -549,7 +544,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   };
 
   settle_loads();
-  tile_pipeline<NS, LPT, LPT>(0, nit, needed, issue, compute);
+  tile_pipeline<NS, LPT, LPT>(0, nit, find, issue, compute);
 
   if (jok) {
     bf16_t *dkp = reinterpret_cast<bf16_t *>(a.dk) + b * a.dk_sb + (int64_t)j * a.dk_ss + hk * a.dk_sh;
@@ -635,14 +630,19 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   if (lane == 0 && pwave) red_s[pair] = kmin_w;
   const int nqt = a.Sq_pad / 64;
   const tile_summary_t *qsum = a.qsum + (int64_t)b * nqt;
-  SummaryTable qtab;
-  qtab.fill(qsum, reinterpret_cast<tile_summary_t *>(smem + L::kBytes + 2 * XBYTES), nqt, tid, NT);
   __syncthreads();
   int kmin_g = kIntMax;
 #pragma unroll
   for (int x = 0; x < NP; ++x) kmin_g = min(kmin_g, red_s[x]);
   kmin_g = __builtin_amdgcn_readfirstlane(kmin_g);  // read from LDS, but the same in every lane
-  const int nit = (kmin_g == kIntMax) ? 0 : a.G * nqt;
+  // A query tile is needed if it has a valid query that sees some key of the workgroup.
+  NeededTable qtab;
+  qtab.fill(qsum, reinterpret_cast<i32x4 *>(smem + L::kBytes + 2 * XBYTES), nqt, tid, NT,
+            [&](const tile_summary_t sm) { return sm.w > 0 && sm.y >= kmin_g; });
+  __syncthreads();
+  // Iterations run over (query head of the group, query tile), head-major; an iteration
+  // index is head << 16 | tile, so neither part needs a division.
+  const int nit = (kmin_g == kIntMax) ? 0 : a.G << 16;
 
   const bf16_t *qb0 = reinterpret_cast<const bf16_t *>(a.q.ptr) + b * a.q.sb + (int64_t)hk * a.G * a.q.sh;
   const bf16_t *gb0 =
@@ -661,38 +661,30 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   gld.init(tid, a.d_o.ss);
   const uint32_t qstep = (uint32_t)(64 * a.q.ss * 2), gstep = (uint32_t)(64 * a.d_o.ss * 2);
 
-  // Iterations run over (query head of the group, query tile), head-major; (head, tile)
-  // follow the iteration index by counting.
-  int at_g = 0, at_base = 0;  // head of the iteration asked about last, and its first iteration
-  auto needed = [&](int it) {
-    int g = at_g, base = at_base;
-    while (it >= base + nqt) base += nqt, ++g;
-    at_g = __builtin_amdgcn_readfirstlane(g);
-    at_base = __builtin_amdgcn_readfirstlane(base);
-    const tile_summary_t sm = qtab.at(it - at_base);
-    return sm.w > 0 && sm.y >= kmin_g;
-  };
+  // first needed iteration at or after `it`: in its head, else the first of the next head
+  // (every head has the same needed tiles)
   auto find = [&](int it) {
-    while (it < nit && !needed(it)) ++it;
-    return __builtin_amdgcn_readfirstlane(it);
+    if (it >= nit) return nit;
+    const int g = it >> 16, qt = it & 0xffff;
+    const int nn = qtab.at(qt < nqt ? qt : nqt).x;
+    int r = (g << 16) | nn;
+    if (nn >= nqt) {
+      const int first = qtab.at(0).x;
+      r = first < nqt ? ((g + 1) << 16) | first : nit;
+    }
+    return __builtin_amdgcn_readfirstlane(r < nit ? r : nit);
   };
-  // summary of an iteration at or before the one asked about last
+  // min id, max id, all-valid flag of a needed iteration's query tile
   auto summary_of = [&](int it) {
-    int qt = it - at_base;
-    while (qt < 0) qt += nqt;
-    return qtab.at(__builtin_amdgcn_readfirstlane(qt));
+    const i32x4 e = qtab.at(it & 0xffff);
+    return tile_summary_t{e.y, e.z, e.w, 0};
   };
   const uint32_t smem0 = lds_addr(smem);
   constexpr int KL = TileLoad<D, NT>::kLoads;
   constexpr int LPT = 2 * KL + 1;  // loads per tile and wave: Q, dO, one statistics row
-  // (head, tile) of the iteration to request: set by locate() before the parts go out,
-  // so that the parts themselves are free of branches
+  // (head, tile) of the iteration to request: set by locate() before the parts go out
   int req_g = 0, req_qt = 0;
-  auto locate = [&](int it) {
-    int g = at_g, qt = it - at_base;  // the head asked about last is this one or a later one: count back
-    while (qt < 0) qt += nqt, --g;
-    req_g = __builtin_amdgcn_readfirstlane(g), req_qt = __builtin_amdgcn_readfirstlane(qt);
-  };
+  auto locate = [&](int it) { req_g = it >> 16, req_qt = it & 0xffff; };
   auto issue = [&](int, auto stage_c, auto part_c, bool live) {
     constexpr int P = decltype(part_c)::value;
     constexpr int S = decltype(stage_c)::value;
@@ -1028,8 +1020,8 @@ template <int D, int NP>
 static int launch_dkv_pair(const BwdArgs &a, hipStream_t st) {
   if (!allow_dynamic_lds<&bwd_dkv_pair_kernel<D, NP>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
   constexpr size_t fixed = dkv_pair_smem_bytes<D, NP>();
-  if (!summary_table_fits(fixed, a.Sq_pad / 64)) return BCATTN_ERR_UNSUPPORTED;
-  const size_t smem = fixed + (size_t)(a.Sq_pad / 64) * sizeof(tile_summary_t);
+  if (!needed_table_fits(fixed, a.Sq_pad / 64)) return BCATTN_ERR_UNSUPPORTED;
+  const size_t smem = fixed + needed_table_bytes(a.Sq_pad / 64);
   const int nkt = (a.Sk + 32 * NP - 1) / (32 * NP);
   hipLaunchKernelGGL((bwd_dkv_pair_kernel<D, NP>), dim3(xcd_grid((unsigned)(nkt * a.Hkv * a.B))),
                      dim3(128 * NP), smem, st, a);
@@ -1044,8 +1036,8 @@ constexpr size_t dkv_smem_bytes() {
 template <int D, int NW, int MODE>
 static int launch_dkv(const BwdArgs &a, hipStream_t st) {
   if (!allow_dynamic_lds<&bwd_dkv_kernel<D, NW, MODE>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
-  if (!summary_table_fits(dkv_smem_bytes<D>(), a.Sq_pad / 64)) return BCATTN_ERR_UNSUPPORTED;
-  const size_t smem = dkv_smem_bytes<D>() + (size_t)(a.Sq_pad / 64) * sizeof(tile_summary_t);
+  if (!needed_table_fits(dkv_smem_bytes<D>(), a.Sq_pad / 64)) return BCATTN_ERR_UNSUPPORTED;
+  const size_t smem = dkv_smem_bytes<D>() + needed_table_bytes(a.Sq_pad / 64);
   const int nkt = (a.Sk + 32 * NW - 1) / (32 * NW);
   hipLaunchKernelGGL((bwd_dkv_kernel<D, NW, MODE>), dim3(xcd_grid((unsigned)(nkt * a.Hkv * a.B))),
                      dim3(64 * NW), smem, st, a);
@@ -1057,7 +1049,7 @@ static int launch_dkv(const BwdArgs &a, hipStream_t st) {
 template <int D, int NWQ, int NWK, bool SPLIT, int PAIRS = 0>
 static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
   if (!allow_dynamic_lds<&bwd_dq_kernel<D, NWQ>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
-  if (!summary_table_fits(dq_smem_bytes<D>(), (a.Sk + 63) / 64)) return BCATTN_ERR_UNSUPPORTED;
+  if (!needed_table_fits(dq_smem_bytes<D>(), (a.Sk + 63) / 64)) return BCATTN_ERR_UNSUPPORTED;
   if (a.stages & BCATTN_BWD_DELTA) {
     constexpr int RPB = 256 / (D / 8);
     const int64_t rows = (int64_t)a.B * a.H * a.Sq_pad;
@@ -1066,7 +1058,7 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
   if (a.stages & BCATTN_BWD_DQ) {
     const int R = a.G * a.Sq;
     const int ntile_r = (R + 32 * NWQ - 1) / (32 * NWQ);
-    const size_t smem = dq_smem_bytes<D>() + (size_t)((a.Sk + 63) / 64) * sizeof(tile_summary_t);
+    const size_t smem = dq_smem_bytes<D>() + needed_table_bytes((a.Sk + 63) / 64);
     hipLaunchKernelGGL((bwd_dq_kernel<D, NWQ>), dim3(xcd_grid((unsigned)(ntile_r * a.Hkv * a.B))), dim3(64 * NWQ),
                        smem, st, a);
   }

@@ -234,13 +234,14 @@ inline bool allow_dynamic_lds(int bytes) {
   return true;
 }
 
-// The tile summaries a workgroup walks are copied to LDS after its tile stages; a
-// sequence with more tiles than fit in the CU's 160 KB is refused by the launcher
-// (more than 100 000 positions at head_dim 256, twice that at 128).
+// The table of needed tiles that a workgroup walks sits in LDS after its tile stages
+// (one 16-byte entry per tile of the row and one more); a sequence with more tiles than
+// fit in the CU's 160 KB is refused by the launcher (more than 100 000 positions at
+// head_dim 256, twice that at 128).
 constexpr size_t kLdsBytes = 160 * 1024;
-inline bool summary_table_fits(size_t stage_bytes, int tiles) {
-  const size_t room = kLdsBytes - 1024 - stage_bytes;  // 1 KB: the kernels' small static arrays
-  return (size_t)tiles * sizeof(tile_summary_t) <= room;
+inline size_t needed_table_bytes(int tiles) { return ((size_t)tiles + 1) * 16; }
+inline bool needed_table_fits(size_t stage_bytes, int tiles) {
+  return needed_table_bytes(tiles) <= kLdsBytes - 1024 - stage_bytes;  // 1 KB: the kernels' small static arrays
 }
 
 // kernel launchers, one translation unit each

@@ -143,8 +143,6 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
     red_s[wave] = qmax_w;
     red_s[NW + wave] = any_w;
   }
-  SummaryTable ktab;
-  ktab.fill(ksum, reinterpret_cast<tile_summary_t *>(smem + L::kBytes), SPLIT ? 0 : nt_all, tid, NT);
   __syncthreads();
   int qmax_g = kIntMin, any_g = 0;
 #pragma unroll
@@ -159,7 +157,13 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   const int nt = !any_g ? 0 : t_last;
   const_summary_t *ksum_s = scalar_view(ksum);
   // A tile is needed if some row of the workgroup can see one of its keys.
-  auto needed = [&](int t) { return ktab.at(t).x <= qmax_g; };
+  NeededTable ktab;
+  if (!SPLIT) {
+    ktab.fill(ksum, reinterpret_cast<i32x4 *>(smem + L::kBytes), nt_all, tid, NT,
+              [&](const tile_summary_t sm) { return sm.x <= qmax_g; });
+    __syncthreads();
+  }
+  auto find = [&](int t) { return ktab.at(t).x; };
   RowAddr<D> rowa;
   rowa.init(lane, smem0);
   TrAddr<D> tra;
@@ -276,11 +280,12 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
     auto issue_part = [&](int t, auto stage_c, auto, bool live) { issue_if(t, stage_c, live); };
     auto compute = [&](auto stage_c, int t, auto bg) {
       bg(StageC<0>{});
-      compute_sm(stage_c, ktab.at(t));
+      const i32x4 e = ktab.at(t);
+      compute_sm(stage_c, tile_summary_t{e.y, e.z, e.w, 0});
       return true;
     };
     settle_loads();
-    tile_pipeline<NS, LPT, 1>(t_first, nt, needed, issue_part, compute);
+    tile_pipeline<NS, LPT, 1>(t_first, nt, find, issue_part, compute);
   }
 
   // ---- epilogue ----------------------------------------------------------------
@@ -406,9 +411,9 @@ template <int D, int NW, bool SPLIT>
 static int launch_fwd_t(const FwdArgs &a, const SplitArgs &sp, hipStream_t st) {
   constexpr size_t stages = fwd_stage_bytes<D, SPLIT>();
   if (!allow_dynamic_lds<&fwd_bf16_kernel<D, NW, SPLIT>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
-  const int tiles = SPLIT ? 0 : (a.Sk0 + 63) / 64 + (a.Sk - a.Sk0 + 63) / 64;
-  if (!summary_table_fits(stages, tiles)) return BCATTN_ERR_UNSUPPORTED;
-  const size_t smem = stages + (size_t)tiles * sizeof(tile_summary_t);
+  const int tiles = (a.Sk0 + 63) / 64 + (a.Sk - a.Sk0 + 63) / 64;
+  if (!SPLIT && !needed_table_fits(stages, tiles)) return BCATTN_ERR_UNSUPPORTED;
+  const size_t smem = stages + (SPLIT ? 0 : needed_table_bytes(tiles));
   const int R = a.G * a.Sq;
   const int ntile_r = (R + 32 * NW - 1) / (32 * NW);
   hipLaunchKernelGGL((fwd_bf16_kernel<D, NW, SPLIT>),

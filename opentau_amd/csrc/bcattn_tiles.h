@@ -267,17 +267,33 @@ __device__ __forceinline__ const_summary_t *scalar_view(const tile_summary_t *p)
   return (const_summary_t *)reinterpret_cast<uintptr_t>(p);
 }
 
-// The summaries of a row of tiles, kept in LDS: a read costs an LDS access instead
-// of a trip to memory, and the main loop holds no ordinary memory load at all (one
+// Which tiles of a row a workgroup needs, kept in LDS: entry i (i = 0..n) describes the
+// first needed tile at or after i as {its index (n if there is none), and its summary's
+// min id, max id, all-valid flag}.  Finding the next tile and reading its summary is one
+// LDS read with no loop, and the main loop holds no ordinary memory load at all (one
 // would be waited for with a count that also drains the asynchronous tile loads).
-struct SummaryTable {
-  const tile_summary_t *lds;
-  // every thread of the workgroup calls this; a barrier must follow before at()
-  __device__ __forceinline__ void fill(const tile_summary_t *src, tile_summary_t *dst, int n, int tid, int nthreads) {
+struct NeededTable {
+  const i32x4 *lds;
+  // Every thread of the workgroup calls this; a barrier must follow before at().
+  // needed(summary) -> bool is the workgroup's test.
+  template <class Pred>
+  __device__ __forceinline__ void fill(const tile_summary_t *src, i32x4 *dst, int n, int tid, int nthreads,
+                                       Pred needed) {
     lds = dst;
-    for (int i = tid; i < n; i += nthreads) dst[i] = src[i];
+    for (int i = tid; i <= n; i += nthreads) {
+      i32x4 e = {n, 0, 0, 0};
+      for (int j = i; j < n; ++j) {
+        const tile_summary_t sm = src[j];
+        if (needed(sm)) {
+          e = i32x4{j, sm.x, sm.y, sm.z};
+          break;
+        }
+      }
+      dst[i] = e;
+    }
   }
-  __device__ __forceinline__ tile_summary_t at(int t) const { return uniform_summary(lds[t]); }
+  // {index of the first needed tile at or after t, min id, max id, all valid}; uniform
+  __device__ __forceinline__ i32x4 at(int t) const { return uniform_summary(lds[t]); }
 };
 
 // Wait for every ordinary load issued so far, in a form the compiler takes note of.
@@ -300,8 +316,8 @@ __device__ __forceinline__ void tile_barrier() { asm volatile("s_barrier" ::: "m
 
 // Walk the needed tiles of [first, end) with NS LDS stages, i.e. NS-1 tiles of
 // prefetch:
-//   needed(t)            does some row of the workgroup use tile t (reads the
-//                        tile's summary from the LDS table)
+//   find(t)              first needed tile at or after t (anything >= end if none; one
+//                        read of the NeededTable)
 //   issue(t, StageC, StageC<part>, live)   requests part `part` of NPARTS of tile t
 //                        into that stage; over all parts every wave must issue
 //                        exactly LPT loads.  With live == false the same loads go
@@ -315,25 +331,12 @@ __device__ __forceinline__ void tile_barrier() { asm volatile("s_barrier" ::: "m
 //                        unit with nothing in flight), one that returns false for none
 // The loop is written out over the stages so that every LDS address inside
 // compute() is a lane offset plus a compile-time constant.  Only tile indices
-// are carried from step to step (scalar registers are scarce in these kernels);
-// the answer for the tile the next search starts at is fetched one step early.
-template <int NS, int LPT, int NPARTS, class Needed, class Issue, class Compute>
-__device__ __forceinline__ void tile_pipeline(int first, int end, Needed needed, Issue issue, Compute compute) {
+// are carried from step to step (scalar registers are scarce in these kernels).
+template <int NS, int LPT, int NPARTS, class Find, class Issue, class Compute>
+__device__ __forceinline__ void tile_pipeline(int first, int end, Find find_at, Issue issue, Compute compute) {
   static_assert(NS == 2 || NS == 3, "two or three stages");
-  int ahead_t = -1;
-  bool ahead_ok = false;
-  // first needed tile at or after t (tile indices are uniform: keep them in scalar registers)
-  auto find = [&](int t) {
-    while (t < end) {
-      if (t == ahead_t ? ahead_ok : needed(t)) break;
-      ++t;
-    }
-    return __builtin_amdgcn_readfirstlane(t);
-  };
-  auto look_ahead = [&](int t) {
-    ahead_t = t;
-    if (t < end) ahead_ok = needed(t);
-  };
+  // (tile indices are uniform: keep them in scalar registers)
+  auto find = [&](int t) { return t < end ? __builtin_amdgcn_readfirstlane(find_at(t)) : end; };
   auto issue_all = [&](int t, auto sc, bool live) {
     static_for<NPARTS>([&](auto part) { issue(t, sc, part, live); });
   };
@@ -345,7 +348,6 @@ __device__ __forceinline__ void tile_pipeline(int first, int end, Needed needed,
     t1 = find(t0 + 1);
     issue_all(t1 < end ? t1 : t0, StageC<1>{}, t1 < end);
   }
-  look_ahead((NS == 3 ? t1 : t0) + 1);
   auto step = [&](auto sc) {
     constexpr int S = decltype(sc)::value;
     constexpr StageC<(S + NS - 1) % NS> into{};
@@ -358,7 +360,6 @@ __device__ __forceinline__ void tile_pipeline(int first, int end, Needed needed,
     }
     tile_barrier();
     const int tn = NS == 2 ? t1 : t2;  // the tile due in this step, if any
-    look_ahead(tn + 1);
     const bool due = tn < end;
     const int tq = due ? tn : t0;
     if (!compute(sc, t0, [&](auto part) { issue(tq, into, part, due); })) issue_all(tq, into, due);
