@@ -78,9 +78,6 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
-#ifdef WAVE_PRIO
-  if (NW == 8 && wave >= 4) __builtin_amdgcn_s_setprio(WAVE_PRIO);
-#endif
 
   const int R = a.G * a.Sq;
   const int ntile_r = (R + BM - 1) / BM;
@@ -155,15 +152,22 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   ktab.fill(ksum, reinterpret_cast<i32x4 *>(smem + L::kBytes), nt_all, tid, NT,
             [&](const tile_summary_t sm) { return sm.x <= qmax_g; });
   __syncthreads();
-  auto find = [&](int t) { return ktab.at(t).x; };
+  auto find = [&](int t) __attribute__((always_inline)) { return ktab.at(t).x; };
   const uint32_t smem0 = lds_addr(smem);
-  auto issue = [&](int t, auto stage_c, auto, bool live) {
+  // A tile is requested one load at a time (part p of LPT): the K loads, the V loads,
+  // then the row of key ids.
+  constexpr int KL = TileLoad<D, NT>::kLoads;
+  constexpr int LPT = 2 * KL + 1;  // loads per tile and wave
+  auto issue = [&](int t, auto stage_c, auto part_c, bool live) __attribute__((always_inline)) {
     constexpr int S = decltype(stage_c)::value;
-    kld.issue(rsrc_if(krs, live), smem0 + L::tile(S, 0), (uint32_t)t * kstep, wave);
-    vld.issue(rsrc_if(vrs, live), smem0 + L::tile(S, 1), (uint32_t)t * vstep, wave);
-    load_row64_dwords(rsrc_if(idrs, live), smem0 + L::aux(S), (uint32_t)t * 256, lane);  // every wave, same data
+    constexpr int P = decltype(part_c)::value;
+    if constexpr (P < KL)
+      kld.template issue_one<P>(rsrc_if(krs, live), smem0 + L::tile(S, 0), (uint32_t)t * kstep, wave);
+    else if constexpr (P < 2 * KL)
+      vld.template issue_one<P - KL>(rsrc_if(vrs, live), smem0 + L::tile(S, 1), (uint32_t)t * vstep, wave);
+    else
+      load_row64_dwords(rsrc_if(idrs, live), smem0 + L::aux(S), (uint32_t)t * 256, lane);  // every wave, same data
   };
-  constexpr int LPT = 2 * TileLoad<D, NT>::kLoads + 1;  // loads per tile and wave
 
   RowAddr<D> rowa;
   rowa.init(lane, smem0);
@@ -177,35 +181,38 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
     for (int x = 0; x < 16; ++x) dq[db][x] = 0.f;
   const float c = a.scale * kLog2e;
 
-  auto compute = [&](auto stage_c, int t, auto bg) {
+  auto compute = [&](auto stage_c, int t, auto bg) __attribute__((always_inline)) {
     const i32x4 e = ktab.at(t);
     const tile_summary_t sm = {e.y, e.z, e.w, 0};
-    if (sm.x > qmax_w) return false;
-    bg(StageC<0>{});  // wave-uniform: no row of this wave sees a key of the tile
+    if (sm.x > qmax_w) return false;  // wave-uniform: no row of this wave sees a key of the tile
     constexpr int S = decltype(stage_c)::value;
     constexpr int Kt = L::tile(S, 0), Vt = L::tile(S, 1);
     const int *kb_s = reinterpret_cast<const int *>(smem + L::aux(S));
     const bool needmask = !(sm.z != 0 && sm.y <= qmin_w);
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb) {
+    static_for<2>([&](auto mb_c) {
+      constexpr int mb = decltype(mb_c)::value;
       f32x16 s, dp;
 #pragma unroll
       for (int x = 0; x < 16; ++x) s[x] = 0.f, dp[x] = 0.f;
       constexpr int KB = 2;  // operand reads issued ahead of the products
-#pragma unroll
-      for (int k0 = 0; k0 < DK; k0 += KB) {
+      static_for<DK / KB>([&](auto b_c) {
+        constexpr int k0 = decltype(b_c)::value * KB;
         bf16x8 fa[KB], fb[KB];
 #pragma unroll
         for (int ks = 0; ks < KB; ++ks) {
           fa[ks] = rowa.template read<Kt>(32 * mb, k0 + ks);
           fb[ks] = rowa.template read<Vt>(32 * mb, k0 + ks);
         }
+        // the loads of the tile due in this step go out between the products of the first half
+        static_for<KB>([&](auto ks_c) {
+          if constexpr (mb == 0) parts_at_slot<k0 + decltype(ks_c)::value, DK, LPT>(bg);
+        });
 #pragma unroll
         for (int ks = 0; ks < KB; ++ks) {
           s = mfma32(fa[ks], qf[k0 + ks], s);
           dp = mfma32(fb[ks], gof[k0 + ks], dp);
         }
-      }
+      });
       float ds[16];
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
@@ -229,13 +236,13 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
 #pragma unroll
         for (int db = 0; db < DB; ++db) dq[db] = mfma32(ka[db], dsb[half], dq[db]);
       }
-    }
+    });
     return true;
   };
 
   // Two LDS stages: while tile t is being used, tile t+1 streams into the other one.
   settle_loads();
-  tile_pipeline<NS, LPT, 1>(0, nt, find, issue, compute);
+  tile_pipeline<NS, LPT, LPT>(0, nt, find, issue, compute);
 
   if (rowok) {
     bf16_t *optr = reinterpret_cast<bf16_t *>(a.dq) + b * a.dq_sb + (int64_t)i * a.dq_ss + h * a.dq_sh;
@@ -262,14 +269,6 @@ constexpr size_t dq_smem_bytes() {
 // launches that each recompute S; this is what fits the register file at
 // head_dim 256, and at 128 it lets two waves share a SIMD).
 constexpr int kModeBoth = 0, kModeDV = 1, kModeDK = 2;
-
-// Spreads `parts` things over `slots` >= parts places in order: the part that belongs at
-// slot s (part p sits at slot p*slots/parts), or -1.
-constexpr int part_at_slot(int s, int slots, int parts) {
-  for (int p = 0; p < parts; ++p)
-    if (p * slots / parts == s) return p;
-  return -1;
-}
 
 template <int D, int NW, int MODE>
 __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
@@ -356,7 +355,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
 
   // first needed iteration at or after `it`: in its head, else the first of the next head
   // (every head has the same needed tiles)
-  auto find = [&](int it) {
+  auto find = [&](int it) __attribute__((always_inline)) {
     const int g = it >> 16, qt = it & 0xffff;
     const int nn = qtab.at(qt < nqt ? qt : nqt).x;
     if (nn < nqt) return (g << 16) | nn;
@@ -369,7 +368,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   constexpr int KL = TileLoad<D, NT>::kLoads;
   constexpr int LPT = 2 * KL + 1;  // loads per tile and wave
   int req_g = 0, req_qt = 0;
-  auto issue = [&](int it, auto stage_c, auto part_c, bool live) {
+  auto issue = [&](int it, auto stage_c, auto part_c, bool live) __attribute__((always_inline)) {
     constexpr int P = decltype(part_c)::value;
     constexpr int S = decltype(stage_c)::value;
     if constexpr (P == 0) req_g = it >> 16, req_qt = it & 0xffff;
@@ -412,7 +411,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   // 0x008 matrix, 0x100 LDS read, 0x002 vector ALU); MASKED is a compile-time copy
   // of "some pair of this tile may be masked", so the common case carries no
   // compare/select at all.
-  auto compute_t = [&](auto stage_c, auto masked_c, auto bg) {
+  auto compute_t = [&](auto stage_c, auto masked_c, auto bg) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_c)::value != 0;
     constexpr int S = decltype(stage_c)::value;
     constexpr int Qt = L::tile(S, 0), Gt = L::tile(S, 1);
@@ -424,7 +423,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
 
     // The loads of the tile due in this step go out one at a time between the products
     // of the two A phases.
-    auto phase_a = [&](auto mb_c) {
+    auto phase_a = [&](auto mb_c) __attribute__((always_inline)) {
       constexpr int mb = decltype(mb_c)::value;
 #pragma unroll
       for (int x = 0; x < 16; ++x) {
@@ -433,13 +432,12 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
       }
       static_for<DK>([&](auto ks_c) {
         constexpr int ks = decltype(ks_c)::value;
-        constexpr int part = part_at_slot(mb * DK + ks, 2 * DK, LPT);
-        if constexpr (part >= 0) bg(StageC<part>{});
+        parts_at_slot<mb * DK + ks, 2 * DK, LPT>(bg);
         s[mb] = mfma32(rowa.template read<Qt>(32 * mb, ks), kf[ks], s[mb]);
         if (WANT_DK) dp[mb] = mfma32(rowa.template read<Gt>(32 * mb, ks), vf[ks], dp[mb]);
       });
     };
-    auto softmax = [&](int mb) {
+    auto softmax = [&](int mb) __attribute__((always_inline)) {
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         float p[8], ds[8];
@@ -464,7 +462,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
         if (WANT_DK) dsb[mb][half] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
       }
     };
-    auto phase_c = [&](int mb) {
+    auto phase_c = [&](int mb) __attribute__((always_inline)) {
 #pragma unroll
       for (int half = 0; half < 2; ++half)
 #pragma unroll
@@ -532,7 +530,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-  auto compute = [&](auto stage_c, int it, auto bg) {
+  auto compute = [&](auto stage_c, int it, auto bg) __attribute__((always_inline)) {
     const i32x4 e = qtab.at(it & 0xffff);
     const tile_summary_t sm = {e.y, e.z, e.w, 0};
     if (sm.y < kmin_w) return false;  // wave-uniform: no key of this wave is seen by the tile
@@ -663,7 +661,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
 
   // first needed iteration at or after `it`: in its head, else the first of the next head
   // (every head has the same needed tiles)
-  auto find = [&](int it) {
+  auto find = [&](int it) __attribute__((always_inline)) {
     if (it >= nit) return nit;
     const int g = it >> 16, qt = it & 0xffff;
     const int nn = qtab.at(qt < nqt ? qt : nqt).x;
@@ -675,7 +673,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
     return __builtin_amdgcn_readfirstlane(r < nit ? r : nit);
   };
   // min id, max id, all-valid flag of a needed iteration's query tile
-  auto summary_of = [&](int it) {
+  auto summary_of = [&](int it) __attribute__((always_inline)) {
     const i32x4 e = qtab.at(it & 0xffff);
     return tile_summary_t{e.y, e.z, e.w, 0};
   };
@@ -684,8 +682,8 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   constexpr int LPT = 2 * KL + 1;  // loads per tile and wave: Q, dO, one statistics row
   // (head, tile) of the iteration to request: set by locate() before the parts go out
   int req_g = 0, req_qt = 0;
-  auto locate = [&](int it) { req_g = it >> 16, req_qt = it & 0xffff; };
-  auto issue = [&](int, auto stage_c, auto part_c, bool live) {
+  auto locate = [&](int it) __attribute__((always_inline)) { req_g = it >> 16, req_qt = it & 0xffff; };
+  auto issue = [&](int, auto stage_c, auto part_c, bool live) __attribute__((always_inline)) {
     constexpr int P = decltype(part_c)::value;
     constexpr int S = decltype(stage_c)::value;
     if constexpr (P < KL) {
@@ -700,7 +698,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
       load_row64_dwords(rsrc_if(strs, live), smem0 + L::aux(S) + stat_dst, row, lane);
     }
   };
-  auto issue_all = [&](int it, auto stage_c, bool live) {
+  auto issue_all = [&](int it, auto stage_c, bool live) __attribute__((always_inline)) {
     locate(it);
     static_for<LPT>([&](auto part) { issue(it, stage_c, part, live); });
   };
@@ -714,7 +712,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   char *xpair = smem + L::kBytes + pair * 2048 + lane * 16;
 
   // The barrier of the exchange must find this wave's LDS writes done.
-  auto exchange_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+  auto exchange_barrier = [&]() __attribute__((always_inline)) { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
   f32x16 acc[DB];  // dV^T (P wave) or dK^T (dS wave)
 #pragma unroll
@@ -734,7 +732,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   // two waves of a SIMD are out of phase as well.
   // CUR / PREV: whether halves h and h-1 exist (the very first half has no h-1).
   auto p_half = [&](auto cur_stage, auto mb_c, auto prev_stage, auto pmb_c, auto xcur_c, auto masked_c, auto cur_c,
-                    auto prev_c, auto bg) {
+                    auto prev_c, auto bg) __attribute__((always_inline)) {
     constexpr int mb = decltype(mb_c)::value, pmb = decltype(pmb_c)::value, xcur = decltype(xcur_c)::value;
     constexpr bool MASKED = decltype(masked_c)::value != 0;
     constexpr bool CUR = decltype(cur_c)::value != 0, PREV = decltype(prev_c)::value != 0;
@@ -746,8 +744,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
     if constexpr (CUR) {
       static_for<DK>([&](auto i_c) {
         constexpr int i = decltype(i_c)::value;
-        constexpr int part = part_at_slot(i, DK, LPT);
-        if constexpr (part >= 0) bg(StageC<part>{});
+        parts_at_slot<i, DK, LPT>(bg);
         s = mfma32(rowa.template read<Qt>(32 * mb, i), frag[i], s);
       });
       constexpr int kAhead = DK < 6 ? DK : 6;
@@ -811,7 +808,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   // P o (dP(h-1) - delta) beside the products of dP(h) (which do not depend on it), then
   // dK(h-1).
   auto ds_half = [&](auto cur_stage, auto mb_c, auto prev_stage, auto pmb_c, auto xcur_c, auto cur_c, auto prev_c,
-                     auto bg) {
+                     auto bg) __attribute__((always_inline)) {
     constexpr int mb = decltype(mb_c)::value, pmb = decltype(pmb_c)::value, xcur = decltype(xcur_c)::value;
     constexpr bool CUR = decltype(cur_c)::value != 0, PREV = decltype(prev_c)::value != 0;
     constexpr int CS = decltype(cur_stage)::value, PS = decltype(prev_stage)::value;
@@ -823,8 +820,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
     if constexpr (CUR)
       static_for<DK>([&](auto i_c) {
         constexpr int i = decltype(i_c)::value;
-        constexpr int part = part_at_slot(i, DK, LPT);
-        if constexpr (part >= 0) bg(StageC<part>{});
+        parts_at_slot<i, DK, LPT>(bg);
         dp = mfma32(rowa.template read<Gt>(32 * mb, i), frag[i], dp);
       });
     else
@@ -878,7 +874,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   // After the last half tile: its accumulating products alone.  The stage of the last
   // tile is only known at run time here, which costs an address add per read but keeps
   // this out of the unrolled loop (one copy, and no second set of accumulators).
-  auto p_last = [&](int stage) {
+  auto p_last = [&](int stage) __attribute__((always_inline)) {
     constexpr int A = L::tile(0, 1) / anchor_spacing<D>();
     const int off = L::tile(0, 1) - A * anchor_spacing<D>() + stage * T::kBytes;
 #pragma unroll
@@ -886,7 +882,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
       acc[i % DB] = mfma32(tra.template read_from<A>(off + 16 * (2 + i / DB) * T::kRowBytes, i % DB), pend[i / DB],
                            acc[i % DB]);
   };
-  auto ds_last = [&](int stage) {
+  auto ds_last = [&](int stage) __attribute__((always_inline)) {
     const float *delta_s = reinterpret_cast<const float *>(smem + L::aux(0) + stage * (3 * 256)) + 64;
     const char *xb = xpair + XBYTES;  // the last half is an odd one
     bf16x8 dsb[2];
@@ -912,11 +908,11 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   };
   auto no_bg = [](auto) {};
   // The loop of one role.  Both roles run the same sequence of barriers.
-  auto run = [&](auto role_c) {
+  auto run = [&](auto role_c) __attribute__((always_inline)) {
     constexpr bool PW = decltype(role_c)::value == 0;
     // Half h of iteration `it` (and the accumulating products of half h-1).
     auto half_step = [&](auto cur_stage, int it, auto mb_c, auto prev_stage, auto pmb_c, auto xcur_c, auto cur_c,
-                         auto prev_c, auto bg) {
+                         auto prev_c, auto bg) __attribute__((always_inline)) {
       if constexpr (PW) {
         bool masked = true;
         if (decltype(cur_c)::value) {
@@ -955,7 +951,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
     // tile t0 in stage S: halves 0 and 1; tile t1 (if any) must have landed before the
     // second barrier; tile t2 is requested after the first, into the stage that the
     // previous tile's last accumulating products (first half step) have then left
-    auto step = [&](auto sc) {
+    auto step = [&](auto sc) __attribute__((always_inline)) {
       constexpr int S = decltype(sc)::value;
       constexpr StageC<(S + NS - 1) % NS> before{};
       constexpr StageC<(S + 2) % NS> into{};

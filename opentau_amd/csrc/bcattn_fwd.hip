@@ -45,9 +45,6 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
-#ifdef WAVE_PRIO
-  if (NW == 8 && wave >= 4) __builtin_amdgcn_s_setprio(WAVE_PRIO);
-#endif
 
   const int R = a.G * a.Sq;
   const int ntile_r = (R + BM - 1) / BM;
@@ -87,19 +84,33 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   v1ld.init(tid, a.v1.ss);
 
   const uint32_t smem0 = lds_addr(smem);
-  auto issue_if = [&](int t, auto stage_c, bool live) {
+  // A tile is requested one load at a time (part p of LPT): the K loads, the V loads,
+  // then the row of key ids.
+  constexpr int KL = TileLoad<D, NT>::kLoads;
+  auto issue_part = [&](int t, auto stage_c, auto part_c, bool live) __attribute__((always_inline)) {
     constexpr int S = decltype(stage_c)::value;
+    constexpr int P = decltype(part_c)::value;
     const uint32_t kt = smem0 + L::tile(S, 0), vt = smem0 + L::tile(S, 1);
-    if (t < nt0) {
-      k0ld.issue(rsrc_if(k0rs, live), kt, (uint32_t)(t * 64 * a.k0.ss * 2), wave);
-      v0ld.issue(rsrc_if(v0rs, live), vt, (uint32_t)(t * 64 * a.v0.ss * 2), wave);
+    const bool seg0 = t < nt0;
+    const int ts = seg0 ? t : t - nt0;  // tile within its key segment
+    if constexpr (P < KL) {
+      if (seg0)
+        k0ld.template issue_one<P>(rsrc_if(k0rs, live), kt, (uint32_t)(ts * 64 * a.k0.ss * 2), wave);
+      else
+        k1ld.template issue_one<P>(rsrc_if(k1rs, live), kt, (uint32_t)(ts * 64 * a.k1.ss * 2), wave);
+    } else if constexpr (P < 2 * KL) {
+      if (seg0)
+        v0ld.template issue_one<P - KL>(rsrc_if(v0rs, live), vt, (uint32_t)(ts * 64 * a.v0.ss * 2), wave);
+      else
+        v1ld.template issue_one<P - KL>(rsrc_if(v1rs, live), vt, (uint32_t)(ts * 64 * a.v1.ss * 2), wave);
     } else {
-      k1ld.issue(rsrc_if(k1rs, live), kt, (uint32_t)((t - nt0) * 64 * a.k1.ss * 2), wave);
-      v1ld.issue(rsrc_if(v1rs, live), vt, (uint32_t)((t - nt0) * 64 * a.v1.ss * 2), wave);
+      load_row64_dwords(rsrc_if(idrs, live), smem0 + L::aux(S), (uint32_t)t * 256, lane);  // every wave, same data
     }
-    load_row64_dwords(rsrc_if(idrs, live), smem0 + L::aux(S), (uint32_t)t * 256, lane);  // every wave, same data
   };
-  auto issue = [&](int t, auto stage_c) { issue_if(t, stage_c, true); };
+  auto issue_if = [&](int t, auto stage_c, bool live) __attribute__((always_inline)) {
+    static_for<2 * KL + 1>([&](auto part) { issue_part(t, stage_c, part, live); });
+  };
+  auto issue = [&](int t, auto stage_c) __attribute__((always_inline)) { issue_if(t, stage_c, true); };
   constexpr int LPT = 2 * TileLoad<D, NT>::kLoads + 1;  // loads per tile and wave
 
   // A split workgroup has only a few tiles, so its start-up latency counts: its first
@@ -163,7 +174,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
               [&](const tile_summary_t sm) { return sm.x <= qmax_g; });
     __syncthreads();
   }
-  auto find = [&](int t) { return ktab.at(t).x; };
+  auto find = [&](int t) __attribute__((always_inline)) { return ktab.at(t).x; };
   RowAddr<D> rowa;
   rowa.init(lane, smem0);
   TrAddr<D> tra;
@@ -179,8 +190,8 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   float l = 0.f;        // this lane half's share of the running sum
   const float c = a.scale * kLog2e;
 
-  auto compute_sm = [&](auto stage_c, const tile_summary_t sm) {
-    if (sm.x > qmax_w) return;  // wave-uniform: no row of this wave sees a key of the tile
+  auto compute_sm = [&](auto stage_c, const tile_summary_t sm, auto bg) __attribute__((always_inline)) {
+    if (sm.x > qmax_w) return false;  // wave-uniform: no row of this wave sees a key of the tile
     constexpr int S = decltype(stage_c)::value;
     constexpr int Kt = L::tile(S, 0), Vt = L::tile(S, 1);
     const int *kb_s = reinterpret_cast<const int *>(smem + L::aux(S));
@@ -193,20 +204,22 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
       for (int x = 0; x < 16; ++x) s[mb][x] = 0.f;
     {
       constexpr int KB = DK < 4 ? DK : 4;
-#pragma unroll
-      for (int k0 = 0; k0 < DK; k0 += KB) {
+      static_for<DK / KB>([&](auto b_c) {
+        constexpr int k0 = decltype(b_c)::value * KB;
         bf16x8 ka0[KB], ka1[KB];
 #pragma unroll
         for (int ks = 0; ks < KB; ++ks) {
           ka0[ks] = rowa.template read<Kt>(0, k0 + ks);
           ka1[ks] = rowa.template read<Kt>(32, k0 + ks);
         }
-#pragma unroll
-        for (int ks = 0; ks < KB; ++ks) {
+        static_for<KB>([&](auto ks_c) {
+          constexpr int ks = decltype(ks_c)::value;
+          // the loads of the tile due in this step go out between these products
+          parts_at_slot<k0 + ks, DK, LPT>(bg);
           s[0] = mfma32(ka0[ks], qf[k0 + ks], s[0]);
           s[1] = mfma32(ka1[ks], qf[k0 + ks], s[1]);
-        }
-      }
+        });
+      });
     }
     const bool needmask = !(sm.z != 0 && sm.y <= qmin_w);
     if (needmask) {
@@ -262,30 +275,28 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
         for (int db = 0; db < DBB; ++db) o[d0 + db] = mfma32(va[db], pb[kk], o[d0 + db]);
       }
     }
+    return true;
   };
 
   if constexpr (SPLIT) {
     // the summary of the next tile is fetched while this one is computed
     tile_summary_t sm_next = ksum_s[min(t_first, nt_all - 1)];
-    auto compute_t = [&](auto stage_c, int t) {
+    auto compute_t = [&](auto stage_c, int t) __attribute__((always_inline)) {
       const tile_summary_t sm = sm_next;
       sm_next = ksum_s[min(t + 1, nt_all - 1)];
-      compute_sm(stage_c, sm);
+      compute_sm(stage_c, sm, [](auto) {});
     };
     settle_loads();
     tile_burst<NS, LPT>(t_first, nt, issue, compute_t);
     wait_async_loads_but<0>();  // the early requests, if no row of the workgroup is valid
   } else {
     // While tile t is being used, the next needed tile(s) stream into the other stage(s).
-    auto issue_part = [&](int t, auto stage_c, auto, bool live) { issue_if(t, stage_c, live); };
-    auto compute = [&](auto stage_c, int t, auto bg) {
-      bg(StageC<0>{});
+    auto compute = [&](auto stage_c, int t, auto bg) __attribute__((always_inline)) {
       const i32x4 e = ktab.at(t);
-      compute_sm(stage_c, tile_summary_t{e.y, e.z, e.w, 0});
-      return true;
+      return compute_sm(stage_c, tile_summary_t{e.y, e.z, e.w, 0}, bg);
     };
     settle_loads();
-    tile_pipeline<NS, LPT, 1>(t_first, nt, find, issue_part, compute);
+    tile_pipeline<NS, LPT, LPT>(t_first, nt, find, issue_part, compute);
   }
 
   // ---- epilogue ----------------------------------------------------------------

@@ -53,7 +53,11 @@ __device__ __forceinline__ buf_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
 // The same descriptor, or (live == false) one over zero bytes: loads through it fetch
 // nothing and deliver zeros.
 __device__ __forceinline__ buf_rsrc_t rsrc_if(buf_rsrc_t r, bool live) {
-  r[2] = live ? r[2] : 0;
+  // (descriptors must sit in scalar registers; the compiler is told again that they can)
+  r[0] = __builtin_amdgcn_readfirstlane(r[0]);
+  r[1] = __builtin_amdgcn_readfirstlane(r[1]);
+  r[2] = __builtin_amdgcn_readfirstlane(live ? r[2] : 0);
+  r[3] = __builtin_amdgcn_readfirstlane(r[3]);
   return r;
 }
 
@@ -313,6 +317,16 @@ __device__ __forceinline__ void wait_async_loads_but() {
 // was already awaited by each wave (wait_async_loads*), and a fence would drain
 // the loads that are meant to stay in flight.
 __device__ __forceinline__ void tile_barrier() { asm volatile("s_barrier" ::: "memory"); }
+
+// Spreads `PARTS` requests over `SLOTS` places in order: at slot S, calls bg(StageC<p>{})
+// for every part p that belongs there (part p sits at slot p*SLOTS/PARTS).
+template <int S, int SLOTS, int PARTS, class Bg>
+__device__ __forceinline__ void parts_at_slot(Bg bg) {
+  static_for<PARTS>([&](auto p_c) {
+    constexpr int p = decltype(p_c)::value;
+    if constexpr (p * SLOTS / PARTS == S) bg(p_c);
+  });
+}
 
 // Walk the needed tiles of [first, end) with NS LDS stages, i.e. NS-1 tiles of
 // prefetch:
