@@ -77,29 +77,37 @@ def main() -> int:
     ws_b = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
     parts = ("fwd", "bwd_delta", "bwd_dq", "bwd_dkv")
 
-    def step(ev=None, ready=True):
-        if ev:
-            ev[0].record()
+    def step(ready=True):
+        """One pass of the hot path: the forward call and the backward call."""
         _, lse = fa.forward_raw(q, k, v, *ids, w.scale, workspace=ws_f, summary_ready=ready, out=out)
-        if ev:
-            ev[1].record()
+        fa.backward_raw(go, q, k, v, out, lse, *ids, w.scale, workspace=ws_b, summary_ready=ready, grads=grads)
+        return lse
+
+    def step_by_kernel(ev):
+        """The same work with the backward's kernels launched one call each, timed apart."""
+        ev[0].record()
+        _, lse = fa.forward_raw(q, k, v, *ids, w.scale, workspace=ws_f, summary_ready=True, out=out)
+        ev[1].record()
         for n, st in enumerate((_loader.BWD_DELTA, _loader.BWD_DQ, _loader.BWD_DKV)):
             fa.backward_raw(go, q, k, v, out, lse, *ids, w.scale, stages=st, workspace=ws_b,
-                            summary_ready=ready, grads=grads)
-            if ev:
-                ev[2 + n].record()
+                            summary_ready=True, grads=grads)
+            ev[2 + n].record()
 
     step(ready=False)  # fills the tile summaries once; the masks do not change between steps
     for _ in range(args.warmup):
         step()
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for s in range(args.steps):
-        step(events[s])
+        step()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
+    # per-kernel durations (HIP events on the stream of the launches), outside the timed region
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
+    for s in range(args.steps):
+        step_by_kernel(events[s])
+    torch.cuda.synchronize()
     part_ms = {p: sum(e[i].elapsed_time(e[i + 1]) for e in events) / args.steps for i, p in enumerate(parts)}
     tflops = 14 * unit / (ms_per_step * 1e-3) / 1e12
 

@@ -17,6 +17,8 @@
 // stores), double buffered; the operand that must be contracted over the
 // sequence axis (K^T, Q^T, dO^T) is read from the same row-major tile with the
 // transposing LDS read.
+#include <mutex>
+
 #include "bcattn_tiles.h"
 
 namespace bcattn {
@@ -1040,6 +1042,33 @@ static int launch_dkv(const BwdArgs &a, hipStream_t st) {
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
 }
 
+// The dQ and the dK/dV kernels are independent, and each leaves part of the chip idle
+// while its last workgroups finish (a workgroup holds most of a CU's LDS, so the grid is
+// a small number of "rounds").  When a call runs both, the dK/dV kernel goes to a side
+// stream that is forked from and joined to the caller's stream by events, and the two
+// kernels' workgroups share the chip.  One side stream and event pair per device, made
+// on first use and kept; default priority; calls on one device take turns using them.
+struct SideStream {
+  hipStream_t stream = nullptr;
+  hipEvent_t fork = nullptr, join = nullptr;
+  std::mutex mu;
+  bool ok = false, tried = false;
+};
+static SideStream *side_stream() {
+  static SideStream per_device[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  SideStream *ss = &per_device[dev];
+  std::lock_guard<std::mutex> lock(ss->mu);
+  if (!ss->tried) {
+    ss->tried = true;
+    ss->ok = hipStreamCreateWithFlags(&ss->stream, hipStreamNonBlocking) == hipSuccess &&
+             hipEventCreateWithFlags(&ss->fork, hipEventDisableTiming) == hipSuccess &&
+             hipEventCreateWithFlags(&ss->join, hipEventDisableTiming) == hipSuccess;
+  }
+  return ss->ok ? ss : nullptr;
+}
+
 // NWQ: waves of the dQ kernel; NWK, SPLIT: waves of the dK/dV kernel and whether it
 // runs as two launches (dV, then dK).
 template <int D, int NWQ, int NWK, bool SPLIT, int PAIRS = 0>
@@ -1051,23 +1080,39 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
     const int64_t rows = (int64_t)a.B * a.H * a.Sq_pad;
     hipLaunchKernelGGL(bwd_prep_kernel<D>, dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, a);
   }
-  if (a.stages & BCATTN_BWD_DQ) {
+  const bool both = (a.stages & BCATTN_BWD_DQ) && (a.stages & BCATTN_BWD_DKV);
+  SideStream *ss = both ? side_stream() : nullptr;
+  std::unique_lock<std::mutex> turn;
+  hipStream_t kst = st;  // stream of the dK/dV kernel
+  if (ss) {
+    turn = std::unique_lock<std::mutex>(ss->mu);
+    if (hipEventRecord(ss->fork, st) == hipSuccess && hipStreamWaitEvent(ss->stream, ss->fork, 0) == hipSuccess)
+      kst = ss->stream;
+    else
+      ss = nullptr;
+  }
+  int rc = BCATTN_OK;
+  if (a.stages & BCATTN_BWD_DKV) {
+    if constexpr (PAIRS > 0) {
+      rc = launch_dkv_pair<D, PAIRS>(a, kst);
+    } else if (SPLIT) {
+      if (!(rc = launch_dkv<D, NWK, kModeDV>(a, kst))) rc = launch_dkv<D, NWK, kModeDK>(a, kst);
+    } else {
+      rc = launch_dkv<D, NWK, kModeBoth>(a, kst);
+    }
+  }
+  if (!rc && (a.stages & BCATTN_BWD_DQ)) {
     const int R = a.G * a.Sq;
     const int ntile_r = (R + 32 * NWQ - 1) / (32 * NWQ);
     const size_t smem = dq_smem_bytes<D>() + needed_table_bytes((a.Sk + 63) / 64);
     hipLaunchKernelGGL((bwd_dq_kernel<D, NWQ>), dim3(xcd_grid((unsigned)(ntile_r * a.Hkv * a.B))), dim3(64 * NWQ),
                        smem, st, a);
   }
-  if (a.stages & BCATTN_BWD_DKV) {
-    int rc;
-    if constexpr (PAIRS > 0) {
-      if ((rc = launch_dkv_pair<D, PAIRS>(a, st))) return rc;
-    } else if (SPLIT) {
-      if ((rc = launch_dkv<D, NWK, kModeDV>(a, st)) || (rc = launch_dkv<D, NWK, kModeDK>(a, st))) return rc;
-    } else if ((rc = launch_dkv<D, NWK, kModeBoth>(a, st))) {
-      return rc;
-    }
+  if (ss) {  // join, whatever happened in between: the caller's stream must not run ahead of the side stream
+    if (hipEventRecord(ss->join, ss->stream) != hipSuccess || hipStreamWaitEvent(st, ss->join, 0) != hipSuccess)
+      rc = rc ? rc : BCATTN_ERR_LAUNCH;
   }
+  if (rc) return rc;
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
 }
 
