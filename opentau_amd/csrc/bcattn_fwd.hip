@@ -239,9 +239,15 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
 #pragma unroll
       for (int x = 0; x < 16; ++x) mloc = fmaxf(mloc, s[mb][x]);
     mloc = fmaxf(mloc, swap32(mloc));
-    const float mnew = fmaxf(m, mloc);
+    // The reference point of the exponentials follows the row maximum only when that has
+    // grown by more than 2^8 (in the exponent): a stale reference leaves P <= 256, which
+    // bf16 and the fp32 sums hold as well as P <= 1, and the accumulators are rescaled
+    // on a few tiles per row instead of on nearly every one.  O / l and the log-sum-exp
+    // do not depend on the reference.
+    const bool grow = (mloc - m) * c > 8.f;  // false for a fully masked tile (mloc = -inf)
+    const float mnew = grow ? mloc : m;
     const float moff = (mnew == -INFINITY) ? 0.f : mnew * c;
-    if (__any(mnew > m)) {
+    if (__any(grow)) {
       const float corr = fast_exp2(m * c - moff);
       l *= corr;
 #pragma unroll
