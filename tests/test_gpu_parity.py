@@ -176,6 +176,26 @@ def test_backward_bf16_cross_attention_non_square():
         assert rel_l2(got, ref) <= 1e-2, name
 
 
+@pytest.mark.parametrize("pattern", PATTERNS)
+@pytest.mark.parametrize("sq,cross,pad_mid", [(300, 0, None), (257, 0, (40, 200)), (129, 190, None)])
+def test_large_group_kernels_head_dim_128(pattern, sq, cross, pad_mid):
+    """G*Sq >= 1024 at head_dim 128 selects the 8-wave forward / dQ kernels and the paired-wave
+    dK/dV kernel (two waves per 32 keys, P exchanged through LDS): ragged last tiles, a padding
+    hole that empties whole key and query tiles, cross attention with a non-square shape."""
+    b, h, hkv, d = 2, 8, 1, 128
+    ids = make_blocks(b, sq, pattern, cross=cross, pad_tail=0 if cross else 9, pad_mid=pad_mid)
+    q, k, v = _qkv(b, sq, cross + sq, h, hkv, d, torch.bfloat16, seed=11)
+    go = randn((b, sq, h, d), torch.bfloat16, 19)
+    scale = d**-0.5
+    out, dq, dk, dv = _fwd_bwd(q, k, v, go, ids, scale)
+    ro, rq, rk, rv = eager.eager_grads(q.float(), k.float(), v.float(), go.float(), *ids, scale)
+    qm = ids[2][:, :, None, None]
+    assert rel_l2(out.float() * qm, ro * qm) <= 1e-2
+    for got, ref, name in ((dq.float() * qm, rq * qm, "dq"), (dk.float(), rk, "dk"), (dv.float(), rv, "dv")):
+        torch.testing.assert_close(got, ref, atol=5e-2, rtol=5e-2)
+        assert rel_l2(got, ref) <= 1e-2, name
+
+
 def test_backward_is_bit_repeatable():
     b, sq, h, hkv, d = 2, 300, 8, 2, 128
     ids = make_blocks(b, sq, "multiblock", pad_tail=17)
