@@ -27,6 +27,17 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0
 
 
+# HBM bytes per launch (fetched + written) of the kernels of the default workload, from two
+# counter runs (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what
+# the same counter reads for a plain 1 GiB device copy (FETCH_SIZE reads half the bytes: factor 2.0;
+# WRITE_SIZE: factor 1.0).  Other workloads have no such measurement and report null.
+HBM_TRAFFIC_BYTES = {
+    ("c5", "fwd"): int((287209.6 * 2.0 + 559482.0) * 1024),
+    ("c5", "bwd_dq"): int((438911.2 * 2.0 + 531897.0) * 1024),
+    ("c5", "bwd_dkv"): int((611929.4 * 2.0 + 70432.0) * 1024),
+}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -34,6 +45,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-denoise", action="store_true", help="skip the pi0.5 denoise leg")
+    ap.add_argument("--serial", action="store_true",
+                    help="keep the backward's two big kernels on one stream (for per-kernel profiles)")
     ap.add_argument("--workload", default="c5", choices=["c3", "c4", "c5"])
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="only run a plain device copy of MIB MiB a few times (reference for the "
@@ -43,6 +56,8 @@ def main() -> int:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
               file=sys.stderr)
         return 2
+    if args.serial:
+        os.environ["BCATTN_SERIAL_BACKWARD"] = "1"  # read by the library when it first runs a backward
 
     import torch
 
@@ -119,12 +134,13 @@ def main() -> int:
     achieved = credit[dom] / (part_ms[dom] * 1e-3) / 1e12
     roofline = {
         "bound": "mfma",
-        "kernel": {"fwd": "fwd_bf16_kernel", "bwd_dq": "bwd_dq_kernel", "bwd_dkv": "bwd_dkv_kernel"}[dom],
+        "kernel": {"fwd": "fwd_bf16_kernel", "bwd_dq": "bwd_dq_kernel",
+                   "bwd_dkv": "bwd_dkv_pair_kernel" if w.D == 128 else "bwd_dkv_kernel"}[dom],
         "achieved": round(achieved, 2),
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-        "traffic": None,
+        "traffic": HBM_TRAFFIC_BYTES.get((w.name, dom)),
         "kernel_ms": {p: round(part_ms[p], 4) for p in parts},
         "kernel_tflops": {p: round(credit[p] / (part_ms[p] * 1e-3) / 1e12, 2) for p in parts if credit[p]},
         "step_frac": round(tflops / PEAK_BF16_TFLOPS, 4),
@@ -252,8 +268,9 @@ def cpu_baseline(torch, make_workload, name, budget_s=12.0):
         pairs_b = int(eager.dense_mask_from_block_ids(*sl).sum())
         for hk in range(w.Hkv):
             hs = slice(hk * grp, (hk + 1) * grp)
-            q, go = w.q[b : b + 1, :, hs], w.d_out[b : b + 1, :, hs]
-            k, v = w.k[b : b + 1, :, hk : hk + 1], w.v[b : b + 1, :, hk : hk + 1]
+            # (fp32 copies: the oracle is the reference's eager arithmetic, not a bf16 CPU kernel)
+            q, go = w.q[b : b + 1, :, hs].float(), w.d_out[b : b + 1, :, hs].float()
+            k, v = w.k[b : b + 1, :, hk : hk + 1].float(), w.v[b : b + 1, :, hk : hk + 1].float()
             t0 = time.perf_counter()
             eager.eager_grads(q, k, v, go, *sl, w.scale)
             dt += time.perf_counter() - t0

@@ -17,6 +17,7 @@
 // stores), double buffered; the operand that must be contracted over the
 // sequence axis (K^T, Q^T, dO^T) is read from the same row-major tile with the
 // transposing LDS read.
+#include <cstdlib>
 #include <mutex>
 
 #include "bcattn_tiles.h"
@@ -183,14 +184,13 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
     for (int x = 0; x < 16; ++x) dq[db][x] = 0.f;
   const float c = a.scale * kLog2e;
 
-  auto compute = [&](auto stage_c, int t, auto bg) __attribute__((always_inline)) {
-    const i32x4 e = ktab.at(t);
-    const tile_summary_t sm = {e.y, e.z, e.w, 0};
-    if (sm.x > qmax_w) return false;  // wave-uniform: no row of this wave sees a key of the tile
+  // MASKED is a compile-time copy of "some pair of this tile may be masked", so that the
+  // common case carries no id reads, compares or selects at all.
+  auto compute_t = [&](auto stage_c, auto masked_c, auto bg) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_c)::value != 0;
     constexpr int S = decltype(stage_c)::value;
     constexpr int Kt = L::tile(S, 0), Vt = L::tile(S, 1);
     const int *kb_s = reinterpret_cast<const int *>(smem + L::aux(S));
-    const bool needmask = !(sm.z != 0 && sm.y <= qmin_w);
     static_for<2>([&](auto mb_c) {
       constexpr int mb = decltype(mb_c)::value;
       f32x16 s, dp;
@@ -219,11 +219,11 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
         i32x4 kb4 = {0, 0, 0, 0};
-        if (needmask) kb4 = *reinterpret_cast<const i32x4 *>(kb_s + 32 * mb + 8 * r4 + 4 * hh);
+        if (MASKED) kb4 = *reinterpret_cast<const i32x4 *>(kb_s + 32 * mb + 8 * r4 + 4 * hh);
 #pragma unroll
         for (int x = 0; x < 4; ++x) {
           float p = fast_exp2(s[4 * r4 + x] * c - lse2);
-          if (needmask && kb4[x] > qb) p = 0.f;
+          if (MASKED && kb4[x] > qb) p = 0.f;
           ds[4 * r4 + x] = p * (dp[4 * r4 + x] - delta);
         }
       }
@@ -239,6 +239,15 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
         for (int db = 0; db < DB; ++db) dq[db] = mfma32(ka[db], dsb[half], dq[db]);
       }
     });
+  };
+  auto compute = [&](auto stage_c, int t, auto bg) __attribute__((always_inline)) {
+    const i32x4 e = ktab.at(t);
+    const tile_summary_t sm = {e.y, e.z, e.w, 0};
+    if (sm.x > qmax_w) return false;  // wave-uniform: no row of this wave sees a key of the tile
+    if (sm.z != 0 && sm.y <= qmin_w)
+      compute_t(stage_c, StageC<0>{}, bg);  // every pair of the tile attends
+    else
+      compute_t(stage_c, StageC<1>{}, bg);
     return true;
   };
 
@@ -1058,6 +1067,13 @@ static SideStream *side_stream() {
   static SideStream per_device[64];
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  // BCATTN_SERIAL_BACKWARD=1 keeps the kernels on the caller's stream, one after the other
+  // (for profiling them apart)
+  static const bool serial = [] {
+    const char *e = getenv("BCATTN_SERIAL_BACKWARD");
+    return e != nullptr && e[0] == '1';
+  }();
+  if (serial) return nullptr;
   SideStream *ss = &per_device[dev];
   std::lock_guard<std::mutex> lock(ss->mu);
   if (!ss->tried) {
