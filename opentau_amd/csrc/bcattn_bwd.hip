@@ -720,7 +720,27 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   tra.init(lane, smem0);
   const float c = a.scale * kLog2e;
   // this pair's part of an exchange buffer: the two 16-query halves of P, 1 KB each
-  char *xpair = smem + L::kBytes + pair * 2048 + lane * 16;
+  // The statistics rows and the exchange buffers sit beyond the 64 KB that an LDS
+  // instruction's immediate reaches: their lane addresses are kept in registers (opaque to
+  // the compiler, like the anchors of the tiles), the rest of each address is an immediate.
+  const int aux_lane = opaque_add(16 * hh, (int)smem0 + L::aux(0));             // statistics of queries 4*hh..
+  const int x_lane = opaque_add(lane * 16 + pair * 2048, (int)smem0 + L::kBytes);  // this lane's exchange slot
+  auto lds_f32x4 = [](int addr) __attribute__((always_inline)) {
+    typedef const __attribute__((address_space(3))) f32x4 T4;
+    return *reinterpret_cast<T4 *>(static_cast<uintptr_t>((uint32_t)addr));
+  };
+  auto lds_i32x4 = [](int addr) __attribute__((always_inline)) {
+    typedef const __attribute__((address_space(3))) i32x4 T4;
+    return *reinterpret_cast<T4 *>(static_cast<uintptr_t>((uint32_t)addr));
+  };
+  auto lds_bf16x8 = [](int addr) __attribute__((always_inline)) {
+    return *reinterpret_cast<lds_bf16x8_t *>(static_cast<uintptr_t>((uint32_t)addr));
+  };
+  auto lds_store_bf16x8 = [](int addr, bf16x8 v) __attribute__((always_inline)) {
+    typedef __attribute__((address_space(3))) bf16x8 T8;
+    *reinterpret_cast<T8 *>(static_cast<uintptr_t>((uint32_t)addr)) = v;
+  };
+
 
   // The barrier of the exchange must find this wave's LDS writes done.
   auto exchange_barrier = [&]() __attribute__((always_inline)) { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
@@ -776,9 +796,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
         acc[i % DB] = mfma32(tra.template read<Gp>(2 * pmb + i / DB, i % DB), pend[i / DB], acc[i % DB]);
       });
     if constexpr (CUR) {
-      const float *lse_s = reinterpret_cast<const float *>(smem + L::aux(CS));
-      const int *qb_s = reinterpret_cast<const int *>(lse_s + 128);
-      char *xb = xpair + xcur * XBYTES;
+      constexpr int AUX = CS * (3 * 256);  // this stage's statistics: lse, delta, ids (256 B each)
       bf16x8 pnew[2];
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
@@ -786,10 +804,9 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
 #pragma unroll
         for (int r2 = 0; r2 < 2; ++r2) {
           const int r4 = 2 * half + r2;
-          const int q0 = 32 * mb + 8 * r4 + 4 * hh;
-          const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lse_s + q0);
+          const f32x4 lse4 = lds_f32x4(aux_lane + AUX + (32 * mb + 8 * r4) * 4);
           i32x4 qb4 = {0, 0, 0, 0};
-          if (MASKED) qb4 = *reinterpret_cast<const i32x4 *>(qb_s + q0);
+          if (MASKED) qb4 = lds_i32x4(aux_lane + AUX + 512 + (32 * mb + 8 * r4) * 4);
 #pragma unroll
           for (int x = 0; x < 4; ++x) {
             float pv = fast_exp2(s[4 * r4 + x] * c - lse4[x]);
@@ -798,7 +815,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
           }
         }
         pnew[half] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
-        *reinterpret_cast<bf16x8 *>(xb + half * 1024) = pnew[half];
+        lds_store_bf16x8(x_lane + xcur * XBYTES + half * 1024, pnew[half]);
       }
       pend[0] = pnew[0], pend[1] = pnew[1];
     }
@@ -837,16 +854,15 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
     else
       static_for<LPT>([&](auto part) { bg(part); });
     if constexpr (PREV) {
-      const float *delta_s = reinterpret_cast<const float *>(smem + L::aux(PS)) + 64;
-      const char *xb = xpair + (1 - xcur) * XBYTES;
+      constexpr int AUX = PS * (3 * 256) + 256;  // delta of the previous half's stage
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
-        const bf16x8 pb = *reinterpret_cast<const bf16x8 *>(xb + half * 1024);
+        const bf16x8 pb = lds_bf16x8(x_lane + (1 - xcur) * XBYTES + half * 1024);
         float ds[8];
 #pragma unroll
         for (int r2 = 0; r2 < 2; ++r2) {
           const int r4 = 2 * half + r2;
-          const f32x4 del4 = *reinterpret_cast<const f32x4 *>(delta_s + 32 * pmb + 8 * r4 + 4 * hh);
+          const f32x4 del4 = lds_f32x4(aux_lane + AUX + (32 * pmb + 8 * r4) * 4);
 #pragma unroll
           for (int x = 0; x < 4; ++x) ds[4 * r2 + x] = (float)pb[4 * r2 + x] * (dp_prev[4 * r4 + x] - del4[x]);
         }
@@ -894,17 +910,16 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
                            acc[i % DB]);
   };
   auto ds_last = [&](int stage) __attribute__((always_inline)) {
-    const float *delta_s = reinterpret_cast<const float *>(smem + L::aux(0) + stage * (3 * 256)) + 64;
-    const char *xb = xpair + XBYTES;  // the last half is an odd one
+    const int aux_stage = aux_lane + stage * (3 * 256) + 256;  // delta of the last tile's stage
     bf16x8 dsb[2];
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
-      const bf16x8 pb = *reinterpret_cast<const bf16x8 *>(xb + half * 1024);
+      const bf16x8 pb = lds_bf16x8(x_lane + XBYTES + half * 1024);  // the last half is an odd one
       float ds[8];
 #pragma unroll
       for (int r2 = 0; r2 < 2; ++r2) {
         const int r4 = 2 * half + r2;
-        const f32x4 del4 = *reinterpret_cast<const f32x4 *>(delta_s + 32 + 8 * r4 + 4 * hh);
+        const f32x4 del4 = lds_f32x4(aux_stage + (32 + 8 * r4) * 4);
 #pragma unroll
         for (int x = 0; x < 4; ++x) ds[4 * r2 + x] = (float)pb[4 * r2 + x] * (dp_prev[4 * r4 + x] - del4[x]);
       }
