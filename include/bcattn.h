@@ -8,9 +8,15 @@
  *     flash_bwd(dO,q,k,v,O,L,q_blk,k_blk,q_valid,k_valid,scale) -> [dQ,dK,dV] (:1210-1327)
  * Here the same two operations, plus a KV-cached variant, are plain C functions
  * over raw device pointers, element strides and an explicit HIP stream.  No
- * torch types, no allocation: the caller owns every buffer (outputs and the
- * workspace), nothing is retained after return, and every call is asynchronous
- * with respect to the host on the stream it is given.
+ * torch types, no device allocation: the caller owns every buffer (outputs and
+ * the workspace), no pointer is retained after return, and every call is
+ * asynchronous with respect to the host on the stream it is given.  The one
+ * thing the library keeps is a helper stream and two events per device, made
+ * on the first bcattn_bwd call that computes all gradients: its two large
+ * kernels run side by side, forked from and joined to the given stream, so
+ * work enqueued on that stream afterwards still sees all of the call's results
+ * (BCATTN_SERIAL_BACKWARD=1 in the environment keeps everything on the given
+ * stream).
  *
  * Mask rule (flash_attn_cuda/__init__.py:27-28):
  *     attend(i,j) = q_valid[i] && k_valid[j] && k_blk[j] <= q_blk[i]
@@ -28,8 +34,11 @@
  * elements (bf16) or 4 elements (fp32).
  *
  * Supported: dtype BCATTN_BF16 with D in {64,128,256} (MFMA kernels) and
- * BCATTN_F32 with D % 32 == 0, D <= 256 (exact fp32 kernels).  Anything else
- * returns BCATTN_ERR_UNSUPPORTED with a message in bcattn_last_error().
+ * BCATTN_F32 with D % 32 == 0, D <= 256 (exact fp32 kernels).  The bf16
+ * kernels index the 64-position tiles of a sequence through a table in LDS,
+ * which bounds the sequence length (about 118 000 positions at D = 256,
+ * 240 000 at D = 128, more at D = 64).  Anything else returns
+ * BCATTN_ERR_UNSUPPORTED with a message in bcattn_last_error().
  */
 #ifndef BCATTN_H_
 #define BCATTN_H_
@@ -48,7 +57,7 @@ enum bcattn_dtype { BCATTN_F32 = 0, BCATTN_BF16 = 1 };
 enum bcattn_status {
   BCATTN_OK = 0,
   BCATTN_ERR_INVALID = -1,     /* null pointer, bad shape, misaligned pointer or stride */
-  BCATTN_ERR_UNSUPPORTED = -2, /* dtype / head_dim the kernels do not cover */
+  BCATTN_ERR_UNSUPPORTED = -2, /* dtype / head_dim / sequence length the kernels do not cover */
   BCATTN_ERR_WORKSPACE = -3,   /* workspace missing or too small */
   BCATTN_ERR_LAUNCH = -4       /* the HIP runtime refused a launch */
 };

@@ -228,6 +228,8 @@ int bcattn_fwd(const bcattn_fwd_params *p, void *stream) {
   char *ws = reinterpret_cast<char *>(p->workspace);
   if ((rc = fwd_prepare(p, a, ws, st))) return rc;
   rc = p->dtype == BCATTN_BF16 ? launch_fwd_bf16(a, p->D, st) : launch_fwd_f32(a, p->D, st);
+  if (rc == BCATTN_ERR_UNSUPPORTED)
+    return fail(rc, "Sk=%d has more 64-key tiles than the kernel's table in LDS holds (D=%d)", p->Sk0 + p->Sk1, p->D);
   if (rc) return fail(rc, "forward launch failed (D=%d dtype=%d)", p->D, p->dtype);
   return BCATTN_OK;
 }
@@ -317,6 +319,9 @@ int bcattn_bwd(const bcattn_bwd_params *p, void *stream) {
        (rc = launch_summary(p->q_blk, p->q_valid, a.B, a.Sq, a.Sq, kIntMin, qs, qm, st))))
     return fail(rc, "summary launch failed");
   rc = p->dtype == BCATTN_BF16 ? launch_bwd_bf16(a, p->D, st) : launch_bwd_f32(a, p->D, st);
+  if (rc == BCATTN_ERR_UNSUPPORTED)
+    return fail(rc, "Sq=%d / Sk=%d have more 64-position tiles than the kernels' tables in LDS hold (D=%d)", p->Sq, p->Sk,
+                p->D);
   if (rc) return fail(rc, "backward launch failed (D=%d dtype=%d)", p->D, p->dtype);
   return BCATTN_OK;
 }

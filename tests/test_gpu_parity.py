@@ -325,6 +325,20 @@ def test_errors_are_raised_not_swallowed():
         fa.forward_raw(k.cpu(), k.cpu(), k.cpu(), *ids, 0.1)
 
 
+def test_sequence_beyond_the_tile_table_is_refused():
+    """The kernels index a sequence's 64-position tiles through a table in LDS; a longer sequence
+    is an error with a message, not a silent fallback."""
+    sk = 130_000  # more tiles than fit beside the two 64 KB stages of head_dim 256
+    q = torch.zeros(1, 8, 1, 256, dtype=torch.bfloat16, device=DEV)
+    k = torch.zeros(1, sk, 1, 256, dtype=torch.bfloat16, device=DEV)
+    q_blk = torch.zeros(1, 8, dtype=torch.int32, device=DEV)
+    k_blk = torch.zeros(1, sk, dtype=torch.int32, device=DEV)
+    q_valid = torch.ones(1, 8, dtype=torch.bool, device=DEV)
+    k_valid = torch.ones(1, sk, dtype=torch.bool, device=DEV)
+    with pytest.raises(RuntimeError, match="tiles"):
+        fa.forward_raw(q, k, k, q_blk, k_blk, q_valid, k_valid, 0.1)
+
+
 # --------------------------------------------------------------------------- #
 # KV-cached suffix call
 # --------------------------------------------------------------------------- #
