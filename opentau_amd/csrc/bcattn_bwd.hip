@@ -439,7 +439,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
 #pragma unroll
       for (int x = 0; x < 16; ++x) {
         s[mb][x] = 0.f;
-        if (WANT_DK) dp[mb][x] = 0.f;
+        if constexpr (WANT_DK) dp[mb][x] = 0.f;
       }
       static_for<DK>([&](auto ks_c) {
         constexpr int ks = decltype(ks_c)::value;

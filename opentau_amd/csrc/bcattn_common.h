@@ -51,11 +51,6 @@ __device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
 
-// Row of the 32x32 accumulator held in register r by a lane of half hh.
-__device__ __forceinline__ constexpr int acc_row(int r, int hh) {
-  return 8 * (r >> 2) + 4 * hh + (r & 3);
-}
-
 // Value held by the lane 32 away (lane ^ 32).
 __device__ __forceinline__ float swap32(float x) {
   return __shfl_xor(x, 32, 64);
@@ -78,12 +73,6 @@ __device__ __forceinline__ int wave_sum_i(int v) {
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
   return v;
 }
-__device__ __forceinline__ float wave_sum_f(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
-}
-
 // Eight fp32 -> eight bf16 (round to nearest even), one MFMA operand.
 __device__ __forceinline__ bf16x8 pack8(float a0, float a1, float a2, float a3, float a4, float a5,
                                         float a6, float a7) {
@@ -111,71 +100,6 @@ __host__ __device__ __forceinline__ unsigned xcd_grid(unsigned n) { return kXcds
 __device__ __forceinline__ int xcd_item(unsigned id, unsigned n) {
   const unsigned chunk = (n + kXcds - 1) / kXcds;
   return (int)((id % kXcds) * chunk + id / kXcds);
-}
-
-// ---------------------------------------------------------------------------
-// LDS layouts.
-//
-// "Row" tiles (keys or queries as rows, head_dim contiguous) are padded by 8
-// elements per row so that a 16-byte read by 16 consecutive rows touches every
-// bank once.
-//
-// "Transposed" tiles hold X^T: one row per head_dim index, 64 sequence
-// positions per row (128 bytes), so that an MFMA operand whose contraction
-// index is the sequence position is one 16-byte read.  Inside a row the 64
-// positions are permuted so that the operand built from a 32x32 accumulator
-// (which gives a lane rows 4*hh..4*hh+3 and 8+4*hh..8+4*hh+3 of each group of 16)
-// meets the matching positions, and 16-byte chunks are XOR-swizzled by the row
-// to keep both the transposing writes and the reads spread over the banks.
-// ---------------------------------------------------------------------------
-template <int D>
-struct RowTile {
-  static constexpr int kPitch = D + 8;
-};
-
-__device__ __forceinline__ int tr_swz(int d) { return ((d >> 1) ^ (d >> 4)) & 7; }
-
-// Element offset, inside a transposed 64-wide row d, of the 16-byte chunk that
-// holds contraction step kk (0..3), lane half hh.
-__device__ __forceinline__ int tr_read_off(int d, int kk, int hh) {
-  return d * 64 + 8 * (((2 * kk + hh)) ^ tr_swz(d));
-}
-
-// Element offset, inside transposed row d, of the 4 consecutive positions
-// 4*kg..4*kg+3 (kg = 0..15) of the 64-wide tile.
-__device__ __forceinline__ int tr_write_off(int d, int kg) {
-  const int chunk = 2 * (kg >> 2) + (kg & 1);
-  const int half = (kg & 3) >> 1;
-  return d * 64 + 8 * (chunk ^ tr_swz(d)) + 4 * half;
-}
-
-// Store a 4(positions) x 8(head_dim) block, given as four 8-wide rows, into the
-// transposed tile: eight 8-byte writes.
-__device__ __forceinline__ void tr_store_4x8(bf16_t *tile, int d0, int kg, bf16x8 r0, bf16x8 r1,
-                                             bf16x8 r2, bf16x8 r3) {
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    bf16x4 w;
-    w[0] = r0[e];
-    w[1] = r1[e];
-    w[2] = r2[e];
-    w[3] = r3[e];
-    *reinterpret_cast<bf16x4 *>(tile + tr_write_off(d0 + e, kg)) = w;
-  }
-}
-
-// Row j of an operand that comes in two segments (n0 rows, then the rest).
-__device__ __forceinline__ const bf16_t *seg_row(const bf16_t *b0, int64_t s0, const bf16_t *b1,
-                                                 int64_t s1, int n0, int j) {
-  return j < n0 ? b0 + (int64_t)j * s0 : b1 + (int64_t)(j - n0) * s1;
-}
-
-// Loads are issued unconditionally from a clamped (always valid) address and
-// zeroed afterwards, so that a tile's loads are all in flight together instead
-// of each sitting in its own branch.
-__device__ __forceinline__ bf16x8 keep_if(bool ok, bf16x8 v) {
-  const bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-  return ok ? v : z;
 }
 
 // ---------------------------------------------------------------------------
@@ -256,20 +180,10 @@ int launch_bwd_f32(const BwdArgs &a, int D, hipStream_t st);
 // Split-key partials of the KV-cached forward.  A work item is (batch, kv head, split,
 // row tile of kSplitRows packed rows); its head_dim accumulators are stored in the order
 // the lanes hold them.
-#ifndef BCATTN_SPLIT_TARGET
-#define BCATTN_SPLIT_TARGET 256
-#endif
-#ifdef BCATTN_PART_BF16
-typedef bf16_t part_t;   // partials normalised by their own sum, so |value| <= max |v|
-typedef bf16x4 part4_t;
-constexpr bool kPartNormalized = true;
-#else
-typedef float part_t;
+typedef float part_t;  // fp32: bf16 partials were measured no faster (the call is latency-bound) and cost accuracy
 typedef f32x4 part4_t;
-constexpr bool kPartNormalized = false;
-#endif
 constexpr int kSplitRows = 128;
-constexpr int kSplitTarget = BCATTN_SPLIT_TARGET;  // workgroups to aim for: one per CU, each holds most of a CU's LDS
+constexpr int kSplitTarget = 256;  // workgroups to aim for: one per CU, each holds most of a CU's LDS
 inline size_t split_ml_bytes(size_t rows) { return (rows * 2 * sizeof(float) + 255) & ~(size_t)255; }
 struct SplitArgs {
   part_t *part_o;  // (B, Hkv, nsplit, row tiles, kSplitRows * D)

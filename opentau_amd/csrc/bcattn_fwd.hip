@@ -320,14 +320,13 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
       *reinterpret_cast<f32x2 *>(sp.part_ml + 2 * (item * BM + wave * 32 + n)) = ml;
     }
     part_t *po = sp.part_o + item * (BM * D) + (int64_t)wave * (32 * D) + 4 * lane;
-    const float pinv = kPartNormalized ? (has ? 1.f / l : 0.f) : 1.f;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
         part4_t w;
 #pragma unroll
-        for (int x = 0; x < 4; ++x) w[x] = (part_t)(o[db][4 * r4 + x] * pinv);
+        for (int x = 0; x < 4; ++x) w[x] = o[db][4 * r4 + x];
         *reinterpret_cast<part4_t *>(po + (db * 4 + r4) * 256) = w;
       }
     return;
@@ -407,10 +406,9 @@ __global__ __launch_bounds__(256) void fwd_combine_kernel(const FwdArgs a, const
       // a split without a visible key has max -inf and sum 0: weight 0, not NaN
       const bool live = s0 + j < sp.nsplit && ml[j][0] != -INFINITY;
       const float e = live ? fast_exp2((ml[j][0] - mref) * c) : 0.f;
-      const float w = kPartNormalized ? e * ml[j][1] : e;
       lsum += e * ml[j][1];
 #pragma unroll
-      for (int x = 0; x < 4; ++x) acc[x] += live ? w * (float)po[j][x] : 0.f;
+      for (int x = 0; x < 4; ++x) acc[x] += live ? e * po[j][x] : 0.f;
     }
   }
   const bool has = lsum > 0.f;
