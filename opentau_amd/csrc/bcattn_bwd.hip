@@ -670,23 +670,24 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   gld.init(tid, a.d_o.ss);
   const uint32_t qstep = (uint32_t)(64 * a.q.ss * 2), gstep = (uint32_t)(64 * a.d_o.ss * 2);
 
-  // first needed iteration at or after `it`: in its head, else the first of the next head
-  // (every head has the same needed tiles)
-  auto find = [&](int it) __attribute__((always_inline)) {
-    if (it >= nit) return nit;
-    const int g = it >> 16, qt = it & 0xffff;
-    const int nn = qtab.at(qt < nqt ? qt : nqt).x;
-    int r = (g << 16) | nn;
-    if (nn >= nqt) {
-      const int first = qtab.at(0).x;
-      r = first < nqt ? ((g + 1) << 16) | first : nit;
-    }
-    return __builtin_amdgcn_readfirstlane(r < nit ? r : nit);
+  // The table entry for iteration `it` (head << 16 | tile), as the lanes read it.  It is asked
+  // for a step before resolve() needs it, so the LDS round trip is off the critical path.
+  auto lookup = [&](int it) __attribute__((always_inline)) {
+    const int qt = it & 0xffff;
+    return qtab.raw(qt < nqt ? qt : nqt);
   };
-  // min id, max id, all-valid flag of a needed iteration's query tile
-  auto summary_of = [&](int it) __attribute__((always_inline)) {
-    const i32x4 e = qtab.at(it & 0xffff);
-    return tile_summary_t{e.y, e.z, e.w, 0};
+  const i32x4 e_first = qtab.at(0);  // first needed tile of a head (every head has the same needed tiles)
+  // First needed iteration at or after `it`, in its head, else the first of the next head;
+  // `masked` tells whether some (query, key) pair of it with this wave's keys is hidden.
+  auto resolve = [&](int it, const i32x4 raw, bool &masked) __attribute__((always_inline)) {
+    i32x4 e = uniform_summary(raw);
+    int r = (it & ~0xffff) | e.x;
+    if (e.x >= nqt) {
+      e = e_first;
+      r = e.x < nqt ? ((it & ~0xffff) + 0x10000) | e.x : nit;
+    }
+    masked = !(e.w != 0 && allk_w != 0 && kmax_w <= e.y);
+    return __builtin_amdgcn_readfirstlane(it < nit && r < nit ? r : nit);
   };
   const uint32_t smem0 = lds_addr(smem);
   constexpr int KL = TileLoad<D, NT>::kLoads;
@@ -937,14 +938,9 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   auto run = [&](auto role_c) __attribute__((always_inline)) {
     constexpr bool PW = decltype(role_c)::value == 0;
     // Half h of iteration `it` (and the accumulating products of half h-1).
-    auto half_step = [&](auto cur_stage, int it, auto mb_c, auto prev_stage, auto pmb_c, auto xcur_c, auto cur_c,
+    auto half_step = [&](auto cur_stage, bool masked, auto mb_c, auto prev_stage, auto pmb_c, auto xcur_c, auto cur_c,
                          auto prev_c, auto bg) __attribute__((always_inline)) {
       if constexpr (PW) {
-        bool masked = true;
-        if (decltype(cur_c)::value) {
-          const tile_summary_t sm = summary_of(it);
-          masked = !(sm.z != 0 && allk_w != 0 && kmax_w <= sm.x);
-        }
         if (masked)
           p_half(cur_stage, mb_c, prev_stage, pmb_c, xcur_c, StageC<1>{}, cur_c, prev_c, bg);
         else  // every pair of the half attends
@@ -953,26 +949,29 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
         ds_half(cur_stage, mb_c, prev_stage, pmb_c, xcur_c, cur_c, prev_c, bg);
       }
     };
-    int t0 = find(0), last_stage = 0;
+    bool m0 = true, m1 = true, m2 = true;  // `masked` of iterations t0, t1, t2
+    int t0 = resolve(0, lookup(0), m0), last_stage = 0;
     if (t0 >= nit) return;
     issue_all(t0, StageC<0>{}, true);
-    int t1 = find(t0 + 1);
+    int t1 = resolve(t0 + 1, lookup(t0 + 1), m1);
     issue_all(t1 < nit ? t1 : t0, StageC<1>{}, t1 < nit);
+    i32x4 ahead = lookup(t1 + 1);
     wait_async_loads_but<LPT>();  // tile t0
     exchange_barrier();
     // very first tile: nothing to accumulate in its first half
     {
-      const int t2 = t1 < nit ? find(t1 + 1) : nit;
-      half_step(StageC<0>{}, t0, StageC<0>{}, StageC<0>{}, StageC<1>{}, StageC<0>{}, StageC<1>{}, StageC<0>{}, no_bg);
+      const int t2 = resolve(t1 + 1, ahead, m2);
+      ahead = lookup(t2 + 1);
+      half_step(StageC<0>{}, m0, StageC<0>{}, StageC<0>{}, StageC<1>{}, StageC<0>{}, StageC<1>{}, StageC<0>{}, no_bg);
       exchange_barrier();  // B(0)
       const bool due = t2 < nit;
       const int tq = due ? t2 : t0;
       locate(tq);
-      half_step(StageC<0>{}, t0, StageC<1>{}, StageC<0>{}, StageC<0>{}, StageC<1>{}, StageC<1>{}, StageC<1>{},
+      half_step(StageC<0>{}, m0, StageC<1>{}, StageC<0>{}, StageC<0>{}, StageC<1>{}, StageC<1>{}, StageC<1>{},
                 [&](auto part) { issue(tq, StageC<2>{}, part, due); });
       wait_async_loads_but<LPT>();  // tile t1
       exchange_barrier();  // B(1)
-      t0 = t1, t1 = t2;
+      t0 = t1, t1 = t2, m0 = m1, m1 = m2;
     }
     // tile t0 in stage S: halves 0 and 1; tile t1 (if any) must have landed before the
     // second barrier; tile t2 is requested after the first, into the stage that the
@@ -985,18 +984,19 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
         last_stage = (S + NS - 1) % NS;
         return true;
       }
-      const int t2 = t1 < nit ? find(t1 + 1) : nit;
+      const int t2 = resolve(t1 + 1, ahead, m2);
+      ahead = lookup(t2 + 1);
       const bool due = t2 < nit;
       const int tq = due ? t2 : t0;
       locate(tq);
       // half 0 of this tile; the accumulating products of half 1 of the previous one
-      half_step(sc, t0, StageC<0>{}, before, StageC<1>{}, StageC<0>{}, StageC<1>{}, StageC<1>{}, no_bg);
+      half_step(sc, m0, StageC<0>{}, before, StageC<1>{}, StageC<0>{}, StageC<1>{}, StageC<1>{}, no_bg);
       exchange_barrier();  // B(2k): half 0's P is there; the previous tile's stage is free
-      half_step(sc, t0, StageC<1>{}, sc, StageC<0>{}, StageC<1>{}, StageC<1>{}, StageC<1>{},
+      half_step(sc, m0, StageC<1>{}, sc, StageC<0>{}, StageC<1>{}, StageC<1>{}, StageC<1>{},
                 [&](auto part) { issue(tq, into, part, due); });
       wait_async_loads_but<LPT>();  // tile t1, for the S / dP of its first half
       exchange_barrier();  // B(2k+1)
-      t0 = t1, t1 = t2;
+      t0 = t1, t1 = t2, m0 = m1, m1 = m2;
       return false;
     };
     for (;;) {

@@ -30,7 +30,7 @@ struct SplitStages {
   static constexpr int value = D <= 128 ? 4 : 2;
 };
 
-template <int D, int NW, bool SPLIT>
+template <int D, int NW, bool SPLIT, bool TWOSEG>
 __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, const SplitArgs sp) {
   using T = Tile<D>;
   constexpr int NT = 64 * NW;   // threads
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
     constexpr int S = decltype(stage_c)::value;
     constexpr int P = decltype(part_c)::value;
     const uint32_t kt = smem0 + L::tile(S, 0), vt = smem0 + L::tile(S, 1);
-    const bool seg0 = t < nt0;
+    const bool seg0 = !TWOSEG || t < nt0;  // one key segment: no choice to make per request
     const int ts = seg0 ? t : t - nt0;  // tile within its key segment
     if constexpr (P < KL) {
       if (seg0)
@@ -422,19 +422,25 @@ __global__ __launch_bounds__(256) void fwd_combine_kernel(const FwdArgs a, const
     a.lse[((int64_t)b * a.H + h) * a.Sq + i] = has ? mx * a.scale + __logf(lsum) : 0.f;
 }
 
-template <int D, int NW, bool SPLIT>
-static int launch_fwd_t(const FwdArgs &a, const SplitArgs &sp, hipStream_t st) {
+// TWOSEG: the keys come as two segments (cache, then new)
+template <int D, int NW, bool SPLIT, bool TWOSEG>
+static int launch_fwd_seg(const FwdArgs &a, const SplitArgs &sp, hipStream_t st) {
   constexpr size_t stages = fwd_stage_bytes<D, SPLIT>();
-  if (!allow_dynamic_lds<&fwd_bf16_kernel<D, NW, SPLIT>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
+  if (!allow_dynamic_lds<&fwd_bf16_kernel<D, NW, SPLIT, TWOSEG>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
   const int tiles = (a.Sk0 + 63) / 64 + (a.Sk - a.Sk0 + 63) / 64;
   if (!SPLIT && !needed_table_fits(stages, tiles)) return BCATTN_ERR_UNSUPPORTED;
   const size_t smem = stages + (SPLIT ? 0 : needed_table_bytes(tiles));
   const int R = a.G * a.Sq;
   const int ntile_r = (R + 32 * NW - 1) / (32 * NW);
-  hipLaunchKernelGGL((fwd_bf16_kernel<D, NW, SPLIT>),
+  hipLaunchKernelGGL((fwd_bf16_kernel<D, NW, SPLIT, TWOSEG>),
                      dim3(xcd_grid((unsigned)(ntile_r * (SPLIT ? sp.nsplit : 1) * a.Hkv * a.B))), dim3(64 * NW),
                      smem, st, a, sp);
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
+}
+
+template <int D, int NW, bool SPLIT>
+static int launch_fwd_t(const FwdArgs &a, const SplitArgs &sp, hipStream_t st) {
+  return a.Sk > a.Sk0 ? launch_fwd_seg<D, NW, SPLIT, true>(a, sp, st) : launch_fwd_seg<D, NW, SPLIT, false>(a, sp, st);
 }
 
 int launch_fwd_bf16(const FwdArgs &a, int D, hipStream_t st) {

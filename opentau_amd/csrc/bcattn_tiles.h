@@ -298,6 +298,9 @@ struct NeededTable {
   }
   // {index of the first needed tile at or after t, min id, max id, all valid}; uniform
   __device__ __forceinline__ i32x4 at(int t) const { return uniform_summary(lds[t]); }
+  // the same entry as the lanes read it (not yet moved to scalar registers): a caller that asks
+  // well before it needs the answer keeps the LDS round trip off its critical path
+  __device__ __forceinline__ i32x4 raw(int t) const { return lds[t]; }
 };
 
 // Wait for every ordinary load issued so far, in a form the compiler takes note of.
