@@ -428,6 +428,93 @@ def test_autograd_op_matches_raw_backward():
 
 
 # --------------------------------------------------------------------------- #
+# how the callers use the op: threads, recompute, tracing
+# --------------------------------------------------------------------------- #
+def test_threads_with_their_own_streams_get_the_serial_results():
+    """The serving path calls the policies from several threads (the reference's
+    ``policies/accel.py:100-104``): concurrent forward+backward calls on separate streams must
+    give, bit for bit, what the same calls give one after the other."""
+    import threading
+
+    b, sq, h, hkv, d = 2, 1100, 16, 2, 128  # long enough for the large-group kernels and the helper stream
+    ids = [g(t) for t in make_blocks(b, sq, "prefixlm", pad_tail=9)]
+    cases = []
+    for t in range(4):
+        q, k, v = (g(x) for x in _qkv(b, sq, sq, h, hkv, d, torch.bfloat16, seed=10 * t))
+        cases.append((q, k, v, g(randn((b, sq, h, d), torch.bfloat16, 10 * t + 7))))
+
+    def run(case):
+        q, k, v, go = case
+        out, lse = fa.forward_raw(q, k, v, *ids, d**-0.5)
+        return (out, *fa.backward_raw(go, q, k, v, out, lse, *ids, d**-0.5))
+
+    serial = [run(c) for c in cases]
+    torch.cuda.synchronize()
+    got, errors = [None] * len(cases), []
+
+    def worker(i):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(3):
+                    got[i] = run(cases[i])
+            stream.synchronize()
+        except Exception as e:  # noqa: BLE001 - reported below
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(cases))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for want, have in zip(serial, got):
+        for a, c in zip(want, have):
+            assert torch.equal(a, c)
+
+
+def test_checkpoint_recompute_gives_the_same_gradients():
+    from torch.utils.checkpoint import checkpoint
+
+    b, sq, h, hkv, d = 2, 90, 8, 1, 256
+    ids = [g(t) for t in make_blocks(b, sq, "prefixlm", pad_tail=4)]
+    q0, k0, v0 = (g(t) for t in _qkv(b, sq, sq, h, hkv, d, torch.bfloat16))
+    go = g(randn((b, sq, h, d), torch.bfloat16, 5))
+
+    def grads(use_checkpoint):
+        q, k, v = (t.clone().requires_grad_(True) for t in (q0, k0, v0))
+        fn = lambda q, k, v: fa.flash_attn_blockmask(q, k, v, *ids, d**-0.5)  # noqa: E731
+        out = checkpoint(fn, q, k, v, use_reentrant=False) if use_checkpoint else fn(q, k, v)
+        out.backward(go)
+        return out.detach(), q.grad, k.grad, v.grad
+
+    for a, c in zip(grads(False), grads(True)):
+        assert torch.equal(a, c)
+
+
+def test_traced_graph_runs_the_same_kernels():
+    """``torch.compile`` traces through the op with its fake implementation and its registered
+    backward (backend ``aot_eager``: the graph is captured and replayed, nothing is generated)."""
+    b, sq, h, hkv, d = 1, 130, 8, 4, 128
+    ids = [g(t) for t in make_blocks(b, sq, "multiblock")]
+    q0, k0, v0 = (g(t) for t in _qkv(b, sq, sq, h, hkv, d, torch.bfloat16))
+    go = g(randn((b, sq, h, d), torch.bfloat16, 5))
+
+    def fn(q, k, v):
+        return fa.flash_attn_blockmask(q * 1.0, k, v, *ids, d**-0.5)
+
+    def grads(f):
+        q, k, v = (t.clone().requires_grad_(True) for t in (q0, k0, v0))
+        out = f(q, k, v)
+        out.backward(go)
+        return out.detach(), q.grad, k.grad, v.grad
+
+    compiled = torch.compile(fn, backend="aot_eager", fullgraph=True)
+    for a, c in zip(grads(fn), grads(compiled)):
+        assert torch.equal(a, c)
+
+
+# --------------------------------------------------------------------------- #
 # the five benchmark configurations
 # --------------------------------------------------------------------------- #
 def test_config1_fp32_forward_full():
