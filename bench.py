@@ -134,7 +134,7 @@ def main() -> int:
     achieved = credit[dom] / (part_ms[dom] * 1e-3) / 1e12
     roofline = {
         "bound": "mfma",
-        "kernel": {"fwd": "fwd_bf16_kernel", "bwd_dq": "bwd_dq_kernel",
+        "kernel": {"fwd": "fwd_mfma_kernel", "bwd_dq": "bwd_dq_kernel",
                    "bwd_dkv": "bwd_dkv_pair_kernel" if w.D == 128 else "bwd_dkv_kernel"}[dom],
         "achieved": round(achieved, 2),
         "peak": PEAK_BF16_TFLOPS,

@@ -31,10 +31,12 @@
  * ELEMENTS, the innermost (head_dim) axis contiguous; so (B,S,H,D), (B,H,S,D)
  * and slices of a preallocated KV cache are all consumed without a copy.  Every
  * base pointer must be 16-byte aligned and every stride a multiple of 8
- * elements (bf16) or 4 elements (fp32).
+ * elements (bf16, fp16) or 4 elements (fp32).
  *
- * Supported: dtype BCATTN_BF16 with D in {64,128,256} (MFMA kernels) and
- * BCATTN_F32 with D % 32 == 0, D <= 256 (exact fp32 kernels).  The bf16
+ * Supported: dtype BCATTN_BF16 or BCATTN_F16 with D in {64,128,256} (MFMA
+ * kernels, fp32 accumulation) and BCATTN_F32 with D % 32 == 0, D <= 256 (exact
+ * fp32 kernels); the reference's kernel takes the same three types
+ * (flash_blockmask.cu:1131, :1142).  The MFMA
  * kernels index the 64-position tiles of a sequence through a table in LDS,
  * which bounds the sequence length (about 118 000 positions at D = 256,
  * 240 000 at D = 128, more at D = 64).  Anything else returns
@@ -52,7 +54,7 @@ extern "C" {
 
 #define BCATTN_ABI_VERSION 1
 
-enum bcattn_dtype { BCATTN_F32 = 0, BCATTN_BF16 = 1 };
+enum bcattn_dtype { BCATTN_F32 = 0, BCATTN_BF16 = 1, BCATTN_F16 = 2 };
 
 enum bcattn_status {
   BCATTN_OK = 0,

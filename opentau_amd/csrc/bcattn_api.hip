@@ -85,8 +85,11 @@ static int check_tensor(const char *name, const bcattn_tensor &t, int vec, bool 
 
 // The MFMA kernels address a (batch, head) slab of an operand through a 32-bit
 // buffer descriptor: rows * stride * 2 bytes must stay below 2^31.
+// bf16 and fp16 run the MFMA kernels
+static bool is16(int dtype) { return dtype == BCATTN_BF16 || dtype == BCATTN_F16; }
+
 static int check_span(const char *name, const bcattn_tensor &t, int rows, int D, int dtype) {
-  if (dtype != BCATTN_BF16 || t.ptr == nullptr) return BCATTN_OK;
+  if (!is16(dtype) || t.ptr == nullptr) return BCATTN_OK;
   if (t.stride_s < D) return fail(BCATTN_ERR_INVALID, "%s: sequence stride smaller than head_dim", name);
   const int64_t bytes = ((int64_t)(rows - 1) * t.stride_s + D) * 2;
   if (bytes >= ((int64_t)1 << 31))
@@ -100,14 +103,14 @@ static int check_common(int B, int Sq, int Sk, int H, int Hkv, int D, int dtype,
     return fail(BCATTN_ERR_INVALID, "bad shape B=%d Sq=%d Sk=%d H=%d Hkv=%d", B, Sq, Sk, H, Hkv);
   if (H % Hkv) return fail(BCATTN_ERR_INVALID, "H=%d is not a multiple of Hkv=%d", H, Hkv);
   if (!(scale > 0.f)) return fail(BCATTN_ERR_INVALID, "scale must be positive");
-  if (dtype == BCATTN_BF16) {
+  if (is16(dtype)) {
     if (D != 64 && D != 128 && D != 256)
-      return fail(BCATTN_ERR_UNSUPPORTED, "bf16 kernels cover head_dim 64, 128, 256; got %d", D);
+      return fail(BCATTN_ERR_UNSUPPORTED, "bf16 / fp16 kernels cover head_dim 64, 128, 256; got %d", D);
   } else if (dtype == BCATTN_F32) {
     if (D % 32 || D <= 0 || D > 256)
       return fail(BCATTN_ERR_UNSUPPORTED, "fp32 kernels need head_dim %% 32 == 0 and <= 256; got %d", D);
   } else {
-    return fail(BCATTN_ERR_UNSUPPORTED, "dtype %d not supported (0 = fp32, 1 = bf16)", dtype);
+    return fail(BCATTN_ERR_UNSUPPORTED, "dtype %d not supported (0 = fp32, 1 = bf16, 2 = fp16)", dtype);
   }
   if ((int64_t)(H / Hkv) * Sq > 0x3fffffff) return fail(BCATTN_ERR_INVALID, "G*Sq too large");
   if ((int64_t)B * H * pad64(Sq) * 4 >= ((int64_t)1 << 31) || (int64_t)B * (Sk + 128) * 4 >= ((int64_t)1 << 31))
@@ -124,7 +127,7 @@ static int check_fwd(const bcattn_fwd_params *p) {
   if (p->Sk0 < 0 || p->Sk1 < 0) return fail(BCATTN_ERR_INVALID, "negative key segment length");
   int rc = check_common(p->B, p->Sq, p->Sk0 + p->Sk1, p->H, p->Hkv, p->D, p->dtype, p->scale);
   if (rc) return rc;
-  const int vec = p->dtype == BCATTN_BF16 ? 8 : 4;
+  const int vec = is16(p->dtype) ? 8 : 4;
   if ((rc = check_tensor("q", p->q, vec, true))) return rc;
   if ((rc = check_tensor("k", p->k, vec, p->Sk0 > 0))) return rc;
   if ((rc = check_tensor("v", p->v, vec, p->Sk0 > 0))) return rc;
@@ -227,7 +230,9 @@ int bcattn_fwd(const bcattn_fwd_params *p, void *stream) {
   FwdArgs a = fwd_args(p);
   char *ws = reinterpret_cast<char *>(p->workspace);
   if ((rc = fwd_prepare(p, a, ws, st))) return rc;
-  rc = p->dtype == BCATTN_BF16 ? launch_fwd_bf16(a, p->D, st) : launch_fwd_f32(a, p->D, st);
+  rc = p->dtype == BCATTN_BF16  ? bf16::launch_fwd_mfma(a, p->D, st)
+       : p->dtype == BCATTN_F16 ? f16::launch_fwd_mfma(a, p->D, st)
+                                : launch_fwd_f32(a, p->D, st);
   if (rc == BCATTN_ERR_UNSUPPORTED)
     return fail(rc, "Sk=%d has more 64-key tiles than the kernel's table in LDS holds (D=%d)", p->Sk0 + p->Sk1, p->D);
   if (rc) return fail(rc, "forward launch failed (D=%d dtype=%d)", p->D, p->dtype);
@@ -238,7 +243,7 @@ int bcattn_fwd_kvcache(const bcattn_fwd_params *p, void *stream) {
   int rc = check_fwd(p);
   if (rc) return rc;
   if (p->B == 0) return BCATTN_OK;
-  if (p->dtype != BCATTN_BF16) return bcattn_fwd(p, stream);
+  if (!is16(p->dtype)) return bcattn_fwd(p, stream);
   const size_t need = bcattn_fwd_kvcache_workspace_bytes(p);
   if (p->workspace == nullptr || p->workspace_bytes < need || !aligned16(p->workspace))
     return fail(BCATTN_ERR_WORKSPACE, "kvcache forward needs %zu bytes of 16-byte aligned workspace, got %zu",
@@ -254,7 +259,8 @@ int bcattn_fwd_kvcache(const bcattn_fwd_params *p, void *stream) {
   const size_t rows = (size_t)a.B * a.Hkv * s.nsplit * ((R + kSplitRows - 1) / kSplitRows) * kSplitRows;
   s.part_ml = reinterpret_cast<float *>(ws);
   s.part_o = reinterpret_cast<part_t *>(ws + split_ml_bytes(rows));
-  rc = launch_fwd_kvcache_bf16(a, s, p->D, st);
+  rc = p->dtype == BCATTN_F16 ? f16::launch_fwd_kvcache_mfma(a, s, p->D, st)
+                              : bf16::launch_fwd_kvcache_mfma(a, s, p->D, st);
   if (rc) return fail(rc, "kvcache forward launch failed (D=%d)", p->D);
   return BCATTN_OK;
 }
@@ -263,7 +269,7 @@ int bcattn_bwd(const bcattn_bwd_params *p, void *stream) {
   if (p == nullptr) return fail(BCATTN_ERR_INVALID, "null params");
   int rc = check_common(p->B, p->Sq, p->Sk, p->H, p->Hkv, p->D, p->dtype, p->scale);
   if (rc) return rc;
-  const int vec = p->dtype == BCATTN_BF16 ? 8 : 4;
+  const int vec = is16(p->dtype) ? 8 : 4;
   const struct {
     const char *n;
     const bcattn_tensor *t;
@@ -318,7 +324,9 @@ int bcattn_bwd(const bcattn_bwd_params *p, void *stream) {
       ((rc = launch_summary(p->k_blk, p->k_valid, a.B, a.Sk, a.Sk, kIntMax, ks, km, st)) ||
        (rc = launch_summary(p->q_blk, p->q_valid, a.B, a.Sq, a.Sq, kIntMin, qs, qm, st))))
     return fail(rc, "summary launch failed");
-  rc = p->dtype == BCATTN_BF16 ? launch_bwd_bf16(a, p->D, st) : launch_bwd_f32(a, p->D, st);
+  rc = p->dtype == BCATTN_BF16  ? bf16::launch_bwd_mfma(a, p->D, st)
+       : p->dtype == BCATTN_F16 ? f16::launch_bwd_mfma(a, p->D, st)
+                                : launch_bwd_f32(a, p->D, st);
   if (rc == BCATTN_ERR_UNSUPPORTED)
     return fail(rc, "Sq=%d / Sk=%d have more 64-position tiles than the kernels' tables in LDS hold (D=%d)", p->Sq, p->Sk,
                 p->D);

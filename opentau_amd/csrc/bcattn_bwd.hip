@@ -23,6 +23,7 @@
 #include "bcattn_tiles.h"
 
 namespace bcattn {
+inline namespace BCATTN_ELEM_NS {
 
 // ---- prep: delta and scaled LSE, padded -------------------------------------------
 template <int D>
@@ -42,9 +43,9 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const BwdArgs a) {
     b = (int)(row / ((int64_t)Sqp * a.H));
     real = i < a.Sq;
     if (real) {
-      const bf16x8 ov = *reinterpret_cast<const bf16x8 *>(reinterpret_cast<const bf16_t *>(a.o.ptr) +
+      const e16x8 ov = *reinterpret_cast<const e16x8 *>(reinterpret_cast<const e16_t *>(a.o.ptr) +
                                                           b * a.o.sb + (int64_t)i * a.o.ss + h * a.o.sh + 8 * c);
-      const bf16x8 gv = *reinterpret_cast<const bf16x8 *>(reinterpret_cast<const bf16_t *>(a.d_o.ptr) +
+      const e16x8 gv = *reinterpret_cast<const e16x8 *>(reinterpret_cast<const e16_t *>(a.d_o.ptr) +
                                                           b * a.d_o.sb + (int64_t)i * a.d_o.ss +
                                                           h * a.d_o.sh + 8 * c);
 #pragma unroll
@@ -102,15 +103,15 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   const bool qv = rowok && a.q_valid[(int64_t)b * a.Sq + i] != 0;
   const int qb = qv ? a.q_blk[(int64_t)b * a.Sq + i] : kIntMin;
 
-  const bf16_t *qptr =
-      reinterpret_cast<const bf16_t *>(a.q.ptr) + b * a.q.sb + (int64_t)i * a.q.ss + h * a.q.sh;
-  const bf16_t *gptr =
-      reinterpret_cast<const bf16_t *>(a.d_o.ptr) + b * a.d_o.sb + (int64_t)i * a.d_o.ss + h * a.d_o.sh;
-  bf16x8 qf[DK], gof[DK];
+  const e16_t *qptr =
+      reinterpret_cast<const e16_t *>(a.q.ptr) + b * a.q.sb + (int64_t)i * a.q.ss + h * a.q.sh;
+  const e16_t *gptr =
+      reinterpret_cast<const e16_t *>(a.d_o.ptr) + b * a.d_o.sb + (int64_t)i * a.d_o.ss + h * a.d_o.sh;
+  e16x8 qf[DK], gof[DK];
 #pragma unroll
   for (int ks = 0; ks < DK; ++ks) {
-    qf[ks] = *reinterpret_cast<const bf16x8 *>(qptr + 16 * ks + 8 * hh);
-    gof[ks] = *reinterpret_cast<const bf16x8 *>(gptr + 16 * ks + 8 * hh);
+    qf[ks] = *reinterpret_cast<const e16x8 *>(qptr + 16 * ks + 8 * hh);
+    gof[ks] = *reinterpret_cast<const e16x8 *>(gptr + 16 * ks + 8 * hh);
   }
   const int64_t stat = ((int64_t)b * a.H + h) * a.Sq_pad + i;
   const float lse2 = rowok ? a.lse2[stat] : INFINITY;  // +inf on rows that take no part
@@ -139,8 +140,8 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   const int Sk = a.Sk;
   const int nt = any_g ? nt_all : 0;
 
-  const bf16_t *kbase = reinterpret_cast<const bf16_t *>(a.k.ptr) + b * a.k.sb + hk * a.k.sh;
-  const bf16_t *vbase = reinterpret_cast<const bf16_t *>(a.v.ptr) + b * a.v.sb + hk * a.v.sh;
+  const e16_t *kbase = reinterpret_cast<const e16_t *>(a.k.ptr) + b * a.k.sb + hk * a.k.sh;
+  const e16_t *vbase = reinterpret_cast<const e16_t *>(a.v.ptr) + b * a.v.sb + hk * a.v.sh;
   const buf_rsrc_t krs = make_rsrc(kbase, (uint32_t)(((int64_t)(Sk - 1) * a.k.ss + D) * 2));
   const buf_rsrc_t vrs = make_rsrc(vbase, (uint32_t)(((int64_t)(Sk - 1) * a.v.ss + D) * 2));
   const buf_rsrc_t idrs =
@@ -199,7 +200,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
       constexpr int KB = 2;  // operand reads issued ahead of the products
       static_for<DK / KB>([&](auto b_c) {
         constexpr int k0 = decltype(b_c)::value * KB;
-        bf16x8 fa[KB], fb[KB];
+        e16x8 fa[KB], fb[KB];
 #pragma unroll
         for (int ks = 0; ks < KB; ++ks) {
           fa[ks] = rowa.template read<Kt>(32 * mb, k0 + ks);
@@ -227,12 +228,12 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
           ds[4 * r4 + x] = p * (dp[4 * r4 + x] - delta);
         }
       }
-      bf16x8 dsb[2];
+      e16x8 dsb[2];
       dsb[0] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
       dsb[1] = pack8(ds[8], ds[9], ds[10], ds[11], ds[12], ds[13], ds[14], ds[15]);
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
-        bf16x8 ka[DB];
+        e16x8 ka[DB];
 #pragma unroll
         for (int db = 0; db < DB; ++db) ka[db] = tra.template read<Kt>(2 * mb + half, db);
 #pragma unroll
@@ -256,15 +257,15 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   tile_pipeline<NS, LPT, LPT>(0, nt, find, issue, compute);
 
   if (rowok) {
-    bf16_t *optr = reinterpret_cast<bf16_t *>(a.dq) + b * a.dq_sb + (int64_t)i * a.dq_ss + h * a.dq_sh;
+    e16_t *optr = reinterpret_cast<e16_t *>(a.dq) + b * a.dq_sb + (int64_t)i * a.dq_ss + h * a.dq_sh;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
-        bf16x4 w;
+        e16x4 w;
 #pragma unroll
-        for (int x = 0; x < 4; ++x) w[x] = (bf16_t)(dq[db][4 * r4 + x] * a.scale);
-        *reinterpret_cast<bf16x4 *>(optr + 32 * db + 8 * r4 + 4 * hh) = w;
+        for (int x = 0; x < 4; ++x) w[x] = (e16_t)(dq[db][4 * r4 + x] * a.scale);
+        *reinterpret_cast<e16x4 *>(optr + 32 * db + 8 * r4 + 4 * hh) = w;
       }
   }
 }
@@ -314,15 +315,15 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   const int jj = jok ? j : Sk - 1;
   const bool kv = jok && a.k_valid[(int64_t)b * Sk + jj] != 0;
   const int kb = kv ? a.k_blk[(int64_t)b * Sk + jj] : kIntMax;
-  const bf16_t *kptr =
-      reinterpret_cast<const bf16_t *>(a.k.ptr) + b * a.k.sb + (int64_t)jj * a.k.ss + hk * a.k.sh;
-  const bf16_t *vptr =
-      reinterpret_cast<const bf16_t *>(a.v.ptr) + b * a.v.sb + (int64_t)jj * a.v.ss + hk * a.v.sh;
-  bf16x8 kf[DK], vf[WANT_DK ? DK : 1];
+  const e16_t *kptr =
+      reinterpret_cast<const e16_t *>(a.k.ptr) + b * a.k.sb + (int64_t)jj * a.k.ss + hk * a.k.sh;
+  const e16_t *vptr =
+      reinterpret_cast<const e16_t *>(a.v.ptr) + b * a.v.sb + (int64_t)jj * a.v.ss + hk * a.v.sh;
+  e16x8 kf[DK], vf[WANT_DK ? DK : 1];
 #pragma unroll
   for (int ks = 0; ks < DK; ++ks) {
-    kf[ks] = *reinterpret_cast<const bf16x8 *>(kptr + 16 * ks + 8 * hh);
-    if (WANT_DK) vf[ks] = *reinterpret_cast<const bf16x8 *>(vptr + 16 * ks + 8 * hh);
+    kf[ks] = *reinterpret_cast<const e16x8 *>(kptr + 16 * ks + 8 * hh);
+    if (WANT_DK) vf[ks] = *reinterpret_cast<const e16x8 *>(vptr + 16 * ks + 8 * hh);
   }
   const int kmin_w = wave_min_i(kb);
   const int kmax_w = wave_max_i(kv ? kb : kIntMin);
@@ -346,9 +347,9 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   // index is head << 16 | tile, so neither part needs a division.
   const int nit = (kmin_g == kIntMax) ? 0 : a.G << 16;
 
-  const bf16_t *qb0 = reinterpret_cast<const bf16_t *>(a.q.ptr) + b * a.q.sb + (int64_t)hk * a.G * a.q.sh;
-  const bf16_t *gb0 =
-      reinterpret_cast<const bf16_t *>(a.d_o.ptr) + b * a.d_o.sb + (int64_t)hk * a.G * a.d_o.sh;
+  const e16_t *qb0 = reinterpret_cast<const e16_t *>(a.q.ptr) + b * a.q.sb + (int64_t)hk * a.G * a.q.sh;
+  const e16_t *gb0 =
+      reinterpret_cast<const e16_t *>(a.d_o.ptr) + b * a.d_o.sb + (int64_t)hk * a.G * a.d_o.sh;
   const uint32_t qbytes = (uint32_t)(((int64_t)(Sq - 1) * a.q.ss + D) * 2);
   const uint32_t gbytes = (uint32_t)(((int64_t)(Sq - 1) * a.d_o.ss + D) * 2);
   const int64_t stat0 = ((int64_t)b * a.H + (int64_t)hk * a.G) * Sqp;  // first row of (b, first head)
@@ -430,7 +431,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
     const float *delta_s = lse_s + 64;
     const int *qb_s = reinterpret_cast<const int *>(delta_s + 64);
     f32x16 s[2], dp[WANT_DK ? 2 : 1];
-    bf16x8 pb[2][2], dsb[2][2];
+    e16x8 pb[2][2], dsb[2][2];
 
     // The loads of the tile due in this step go out one at a time between the products
     // of the two A phases.
@@ -556,20 +557,20 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   tile_pipeline<NS, LPT, LPT>(0, nit, find, issue, compute);
 
   if (jok) {
-    bf16_t *dkp = reinterpret_cast<bf16_t *>(a.dk) + b * a.dk_sb + (int64_t)j * a.dk_ss + hk * a.dk_sh;
-    bf16_t *dvp = reinterpret_cast<bf16_t *>(a.dv) + b * a.dv_sb + (int64_t)j * a.dv_ss + hk * a.dv_sh;
+    e16_t *dkp = reinterpret_cast<e16_t *>(a.dk) + b * a.dk_sb + (int64_t)j * a.dk_ss + hk * a.dk_sh;
+    e16_t *dvp = reinterpret_cast<e16_t *>(a.dv) + b * a.dv_sb + (int64_t)j * a.dv_ss + hk * a.dv_sh;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
-        bf16x4 wk, wv;
+        e16x4 wk, wv;
 #pragma unroll
         for (int x = 0; x < 4; ++x) {
-          if (WANT_DK) wk[x] = (bf16_t)(dk[db][4 * r4 + x] * a.scale);
-          if (WANT_DV) wv[x] = (bf16_t)dv[db][4 * r4 + x];
+          if (WANT_DK) wk[x] = (e16_t)(dk[db][4 * r4 + x] * a.scale);
+          if (WANT_DV) wv[x] = (e16_t)dv[db][4 * r4 + x];
         }
-        if (WANT_DK) *reinterpret_cast<bf16x4 *>(dkp + 32 * db + 8 * r4 + 4 * hh) = wk;
-        if (WANT_DV) *reinterpret_cast<bf16x4 *>(dvp + 32 * db + 8 * r4 + 4 * hh) = wv;
+        if (WANT_DK) *reinterpret_cast<e16x4 *>(dkp + 32 * db + 8 * r4 + 4 * hh) = wk;
+        if (WANT_DV) *reinterpret_cast<e16x4 *>(dvp + 32 * db + 8 * r4 + 4 * hh) = wv;
       }
   }
 }
@@ -629,10 +630,10 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   const int kb = kv ? a.k_blk[(int64_t)b * Sk + jj] : kIntMax;
   // K fragments in the P wave, V fragments in the dS wave
   const bcattn::TensorArg &src = pwave ? a.k : a.v;
-  const bf16_t *fptr = reinterpret_cast<const bf16_t *>(src.ptr) + b * src.sb + (int64_t)jj * src.ss + hk * src.sh;
-  bf16x8 frag[DK];
+  const e16_t *fptr = reinterpret_cast<const e16_t *>(src.ptr) + b * src.sb + (int64_t)jj * src.ss + hk * src.sh;
+  e16x8 frag[DK];
 #pragma unroll
-  for (int ks = 0; ks < DK; ++ks) frag[ks] = *reinterpret_cast<const bf16x8 *>(fptr + 16 * ks + 8 * hh);
+  for (int ks = 0; ks < DK; ++ks) frag[ks] = *reinterpret_cast<const e16x8 *>(fptr + 16 * ks + 8 * hh);
   const int kmin_w = wave_min_i(kb);
   const int kmax_w = wave_max_i(kv ? kb : kIntMin);
   const int allk_w = wave_min_i(kv ? 1 : 0);
@@ -653,9 +654,9 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   // index is head << 16 | tile, so neither part needs a division.
   const int nit = (kmin_g == kIntMax) ? 0 : a.G << 16;
 
-  const bf16_t *qb0 = reinterpret_cast<const bf16_t *>(a.q.ptr) + b * a.q.sb + (int64_t)hk * a.G * a.q.sh;
-  const bf16_t *gb0 =
-      reinterpret_cast<const bf16_t *>(a.d_o.ptr) + b * a.d_o.sb + (int64_t)hk * a.G * a.d_o.sh;
+  const e16_t *qb0 = reinterpret_cast<const e16_t *>(a.q.ptr) + b * a.q.sb + (int64_t)hk * a.G * a.q.sh;
+  const e16_t *gb0 =
+      reinterpret_cast<const e16_t *>(a.d_o.ptr) + b * a.d_o.sb + (int64_t)hk * a.G * a.d_o.sh;
   const uint32_t qbytes = (uint32_t)(((int64_t)(Sq - 1) * a.q.ss + D) * 2);
   const uint32_t gbytes = (uint32_t)(((int64_t)(Sq - 1) * a.d_o.ss + D) * 2);
   const int64_t stat0 = ((int64_t)b * a.H + (int64_t)hk * a.G) * Sqp;
@@ -734,11 +735,11 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
     typedef const __attribute__((address_space(3))) i32x4 T4;
     return *reinterpret_cast<T4 *>(static_cast<uintptr_t>((uint32_t)addr));
   };
-  auto lds_bf16x8 = [](int addr) __attribute__((always_inline)) {
-    return *reinterpret_cast<lds_bf16x8_t *>(static_cast<uintptr_t>((uint32_t)addr));
+  auto lds_e16x8 = [](int addr) __attribute__((always_inline)) {
+    return *reinterpret_cast<lds_e16x8_t *>(static_cast<uintptr_t>((uint32_t)addr));
   };
-  auto lds_store_bf16x8 = [](int addr, bf16x8 v) __attribute__((always_inline)) {
-    typedef __attribute__((address_space(3))) bf16x8 T8;
+  auto lds_store_e16x8 = [](int addr, e16x8 v) __attribute__((always_inline)) {
+    typedef __attribute__((address_space(3))) e16x8 T8;
     *reinterpret_cast<T8 *>(static_cast<uintptr_t>((uint32_t)addr)) = v;
   };
 
@@ -754,7 +755,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
 
   // State carried from one half tile to the next: what the accumulating products of the
   // previous half still need.
-  bf16x8 pend[2] = {};  // P wave: P(h-1) as bf16
+  e16x8 pend[2] = {};  // P wave: P(h-1) as bf16
   f32x16 dp_prev = {};  // dS wave: dP(h-1)
 
   // One half tile of the P wave: S(h) (a chain of dependent products), then softmax(h)
@@ -798,7 +799,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
       });
     if constexpr (CUR) {
       constexpr int AUX = CS * (3 * 256);  // this stage's statistics: lse, delta, ids (256 B each)
-      bf16x8 pnew[2];
+      e16x8 pnew[2];
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         float p[8];
@@ -816,7 +817,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
           }
         }
         pnew[half] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
-        lds_store_bf16x8(x_lane + xcur * XBYTES + half * 1024, pnew[half]);
+        lds_store_e16x8(x_lane + xcur * XBYTES + half * 1024, pnew[half]);
       }
       pend[0] = pnew[0], pend[1] = pnew[1];
     }
@@ -842,7 +843,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
     constexpr bool CUR = decltype(cur_c)::value != 0, PREV = decltype(prev_c)::value != 0;
     constexpr int CS = decltype(cur_stage)::value, PS = decltype(prev_stage)::value;
     constexpr int Gt = L::tile(CS, 1), Qp = L::tile(PS, 0);
-    bf16x8 dsb[2] = {};
+    e16x8 dsb[2] = {};
     f32x16 dp;
 #pragma unroll
     for (int x = 0; x < 16; ++x) dp[x] = 0.f;
@@ -858,7 +859,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
       constexpr int AUX = PS * (3 * 256) + 256;  // delta of the previous half's stage
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
-        const bf16x8 pb = lds_bf16x8(x_lane + (1 - xcur) * XBYTES + half * 1024);
+        const e16x8 pb = lds_e16x8(x_lane + (1 - xcur) * XBYTES + half * 1024);
         float ds[8];
 #pragma unroll
         for (int r2 = 0; r2 < 2; ++r2) {
@@ -912,10 +913,10 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   };
   auto ds_last = [&](int stage) __attribute__((always_inline)) {
     const int aux_stage = aux_lane + stage * (3 * 256) + 256;  // delta of the last tile's stage
-    bf16x8 dsb[2];
+    e16x8 dsb[2];
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
-      const bf16x8 pb = lds_bf16x8(x_lane + XBYTES + half * 1024);  // the last half is an odd one
+      const e16x8 pb = lds_e16x8(x_lane + XBYTES + half * 1024);  // the last half is an odd one
       float ds[8];
 #pragma unroll
       for (int r2 = 0; r2 < 2; ++r2) {
@@ -1018,17 +1019,17 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
     run(StageC<1>{});
 
   if (jok) {
-    bf16_t *dst = pwave ? reinterpret_cast<bf16_t *>(a.dv) + b * a.dv_sb + (int64_t)j * a.dv_ss + hk * a.dv_sh
-                        : reinterpret_cast<bf16_t *>(a.dk) + b * a.dk_sb + (int64_t)j * a.dk_ss + hk * a.dk_sh;
+    e16_t *dst = pwave ? reinterpret_cast<e16_t *>(a.dv) + b * a.dv_sb + (int64_t)j * a.dv_ss + hk * a.dv_sh
+                        : reinterpret_cast<e16_t *>(a.dk) + b * a.dk_sb + (int64_t)j * a.dk_ss + hk * a.dk_sh;
     const float mul = pwave ? 1.f : a.scale;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
-        bf16x4 w;
+        e16x4 w;
 #pragma unroll
-        for (int x = 0; x < 4; ++x) w[x] = (bf16_t)(acc[db][4 * r4 + x] * mul);
-        *reinterpret_cast<bf16x4 *>(dst + 32 * db + 8 * r4 + 4 * hh) = w;
+        for (int x = 0; x < 4; ++x) w[x] = (e16_t)(acc[db][4 * r4 + x] * mul);
+        *reinterpret_cast<e16x4 *>(dst + 32 * db + 8 * r4 + 4 * hh) = w;
       }
   }
 }
@@ -1147,7 +1148,7 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
 }
 
-int launch_bwd_bf16(const BwdArgs &a, int D, hipStream_t st) {
+int launch_bwd_mfma(const BwdArgs &a, int D, hipStream_t st) {
   const int R = a.G * a.Sq;
   switch (D) {
     case 64:
@@ -1161,4 +1162,5 @@ int launch_bwd_bf16(const BwdArgs &a, int D, hipStream_t st) {
   }
 }
 
+}  // namespace BCATTN_ELEM_NS
 }  // namespace bcattn

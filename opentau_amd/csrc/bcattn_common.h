@@ -9,10 +9,19 @@
 
 namespace bcattn {
 
-typedef __bf16 bf16_t;
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+// The MFMA kernels are compiled once per 16-bit element type (bf16, and fp16 with
+// BCATTN_ELEM_F16 defined).  What depends on the element type lives in an inline namespace
+// named after it, so the two sets of kernels and launchers are distinct symbols.
+#ifdef BCATTN_ELEM_F16
+#define BCATTN_ELEM_NS f16
+typedef _Float16 e16_t;
+#else
+#define BCATTN_ELEM_NS bf16
+typedef __bf16 e16_t;
+#endif
+typedef e16_t e16x2 __attribute__((ext_vector_type(2)));
+typedef e16_t e16x4 __attribute__((ext_vector_type(4)));
+typedef e16_t e16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -44,13 +53,6 @@ __device__ __forceinline__ tile_summary_t uniform_summary(tile_summary_t s) {
   return r;
 }
 
-// D(32x32 fp32) += A(32x16 bf16) * B(16x32 bf16).
-// Lane l supplies A[row l%32][k 8*(l/32)..+7] and B[k 8*(l/32)..+7][col l%32];
-// it receives D[row 8*(r/4) + 4*(l/32) + r%4][col l%32] in register r.
-__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-}
-
 // Value held by the lane 32 away (lane ^ 32).
 __device__ __forceinline__ float swap32(float x) {
   return __shfl_xor(x, 32, 64);
@@ -73,20 +75,33 @@ __device__ __forceinline__ int wave_sum_i(int v) {
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
   return v;
 }
-// Eight fp32 -> eight bf16 (round to nearest even), one MFMA operand.
-__device__ __forceinline__ bf16x8 pack8(float a0, float a1, float a2, float a3, float a4, float a5,
+inline namespace BCATTN_ELEM_NS {
+// D(32x32 fp32) += A(32x16) * B(16x32), 16-bit operands.
+// Lane l supplies A[row l%32][k 8*(l/32)..+7] and B[k 8*(l/32)..+7][col l%32];
+// it receives D[row 8*(r/4) + 4*(l/32) + r%4][col l%32] in register r.
+__device__ __forceinline__ f32x16 mfma32(e16x8 a, e16x8 b, f32x16 c) {
+#ifdef BCATTN_ELEM_F16
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+#else
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+#endif
+}
+
+// Eight fp32 -> eight 16-bit elements (round to nearest even), one MFMA operand.
+__device__ __forceinline__ e16x8 pack8(float a0, float a1, float a2, float a3, float a4, float a5,
                                         float a6, float a7) {
-  bf16x8 r;
-  r[0] = (bf16_t)a0;
-  r[1] = (bf16_t)a1;
-  r[2] = (bf16_t)a2;
-  r[3] = (bf16_t)a3;
-  r[4] = (bf16_t)a4;
-  r[5] = (bf16_t)a5;
-  r[6] = (bf16_t)a6;
-  r[7] = (bf16_t)a7;
+  e16x8 r;
+  r[0] = (e16_t)a0;
+  r[1] = (e16_t)a1;
+  r[2] = (e16_t)a2;
+  r[3] = (e16_t)a3;
+  r[4] = (e16_t)a4;
+  r[5] = (e16_t)a5;
+  r[6] = (e16_t)a6;
+  r[7] = (e16_t)a7;
   return r;
 }
+}  // namespace BCATTN_ELEM_NS
 
 // Workgroup -> work item map that keeps neighbours on one XCD.  The hardware
 // hands consecutive workgroup ids to the 8 XCDs in turn, each with its own L2;
@@ -172,9 +187,7 @@ inline bool needed_table_fits(size_t stage_bytes, int tiles) {
 // Tile summaries and merged ids of a sequence given as two segments (n0 rows, then S - n0).
 int launch_summary(const int32_t *blk, const uint8_t *valid, int B, int n0, int S, int fill,
                    tile_summary_t *sum, int32_t *merged, hipStream_t st);
-int launch_fwd_bf16(const FwdArgs &a, int D, hipStream_t st);
 int launch_fwd_f32(const FwdArgs &a, int D, hipStream_t st);
-int launch_bwd_bf16(const BwdArgs &a, int D, hipStream_t st);
 int launch_bwd_f32(const BwdArgs &a, int D, hipStream_t st);
 
 // Split-key partials of the KV-cached forward.  A work item is (batch, kv head, split,
@@ -191,7 +204,27 @@ struct SplitArgs {
   int nsplit;
   int tiles_per_split;  // 64-key tiles per split
 };
-int launch_fwd_kvcache_bf16(const FwdArgs &a, const SplitArgs &s, int D, hipStream_t st);
-size_t kvcache_workspace_bytes(int B, int Sq, int Sk0, int Sk, int H, int Hkv, int D, int *nsplit_out);
+// Launchers of the MFMA kernels, one set per element type (the workspace size of the
+// KV-cached call does not depend on the type; each set carries its copy).
+#define BCATTN_DECLARE_MFMA_LAUNCHERS                                                        \
+  int launch_fwd_mfma(const FwdArgs &a, int D, hipStream_t st);                              \
+  int launch_bwd_mfma(const BwdArgs &a, int D, hipStream_t st);                              \
+  int launch_fwd_kvcache_mfma(const FwdArgs &a, const SplitArgs &s, int D, hipStream_t st);  \
+  size_t kvcache_workspace_bytes(int B, int Sq, int Sk0, int Sk, int H, int Hkv, int D, int *nsplit_out);
+#ifdef BCATTN_ELEM_F16
+inline namespace f16 {
+BCATTN_DECLARE_MFMA_LAUNCHERS
+}
+namespace bf16 {
+BCATTN_DECLARE_MFMA_LAUNCHERS
+}
+#else
+inline namespace bf16 {
+BCATTN_DECLARE_MFMA_LAUNCHERS
+}
+namespace f16 {
+BCATTN_DECLARE_MFMA_LAUNCHERS
+}
+#endif
 
 }  // namespace bcattn

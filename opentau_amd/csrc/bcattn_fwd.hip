@@ -13,6 +13,7 @@
 #include "bcattn_tiles.h"
 
 namespace bcattn {
+inline namespace BCATTN_ELEM_NS {
 
 //
 // SPLIT: the key tiles are divided over `nsplit` workgroups per row tile; each
@@ -31,7 +32,7 @@ struct SplitStages {
 };
 
 template <int D, int NW, bool SPLIT, bool TWOSEG>
-__global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, const SplitArgs sp) {
+__global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, const SplitArgs sp) {
   using T = Tile<D>;
   constexpr int NT = 64 * NW;   // threads
   constexpr int BM = 32 * NW;   // packed query rows per workgroup
@@ -66,10 +67,10 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   const int t_first = SPLIT ? split * sp.tiles_per_split : 0;
   const tile_summary_t *ksum = a.ksum + (int64_t)b * nt_all;
 
-  const bf16_t *k0b = reinterpret_cast<const bf16_t *>(a.k0.ptr) + b * a.k0.sb + hk * a.k0.sh;
-  const bf16_t *v0b = reinterpret_cast<const bf16_t *>(a.v0.ptr) + b * a.v0.sb + hk * a.v0.sh;
-  const bf16_t *k1b = reinterpret_cast<const bf16_t *>(a.k1.ptr) + b * a.k1.sb + hk * a.k1.sh;
-  const bf16_t *v1b = reinterpret_cast<const bf16_t *>(a.v1.ptr) + b * a.v1.sb + hk * a.v1.sh;
+  const e16_t *k0b = reinterpret_cast<const e16_t *>(a.k0.ptr) + b * a.k0.sb + hk * a.k0.sh;
+  const e16_t *v0b = reinterpret_cast<const e16_t *>(a.v0.ptr) + b * a.v0.sb + hk * a.v0.sh;
+  const e16_t *k1b = reinterpret_cast<const e16_t *>(a.k1.ptr) + b * a.k1.sb + hk * a.k1.sh;
+  const e16_t *v1b = reinterpret_cast<const e16_t *>(a.v1.ptr) + b * a.v1.sb + hk * a.v1.sh;
   const int n0 = a.Sk0 > 0 ? a.Sk0 : 1, n1 = a.Sk - a.Sk0 > 0 ? a.Sk - a.Sk0 : 1;
   const buf_rsrc_t k0rs = make_rsrc(k0b, (uint32_t)(((int64_t)(n0 - 1) * a.k0.ss + D) * 2));
   const buf_rsrc_t v0rs = make_rsrc(v0b, (uint32_t)(((int64_t)(n0 - 1) * a.v0.ss + D) * 2));
@@ -139,12 +140,12 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   const bool qv = rowok && qv_raw != 0;
   const int qb = qv ? qb_raw : kIntMin;
 
-  const bf16_t *qptr =
-      reinterpret_cast<const bf16_t *>(a.q.ptr) + b * a.q.sb + (int64_t)i * a.q.ss + h * a.q.sh;
-  bf16x8 qf[DK];
+  const e16_t *qptr =
+      reinterpret_cast<const e16_t *>(a.q.ptr) + b * a.q.sb + (int64_t)i * a.q.ss + h * a.q.sh;
+  e16x8 qf[DK];
 #pragma unroll
   for (int ks = 0; ks < DK; ++ks)
-    qf[ks] = *reinterpret_cast<const bf16x8 *>(qptr + 16 * ks + 8 * hh);
+    qf[ks] = *reinterpret_cast<const e16x8 *>(qptr + 16 * ks + 8 * hh);
 
   // ---- block-id range of the wave and of the workgroup ------------------------
   const int qmax_w = wave_max_i(qv ? qb : kIntMin);
@@ -206,7 +207,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
       constexpr int KB = DK < 4 ? DK : 4;
       static_for<DK / KB>([&](auto b_c) {
         constexpr int k0 = decltype(b_c)::value * KB;
-        bf16x8 ka0[KB], ka1[KB];
+        e16x8 ka0[KB], ka1[KB];
 #pragma unroll
         for (int ks = 0; ks < KB; ++ks) {
           ka0[ks] = rowa.template read<Kt>(0, k0 + ks);
@@ -256,7 +257,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
         for (int x = 0; x < 16; ++x) o[db][x] *= corr;
     }
     m = mnew;
-    bf16x8 pb[4];
+    e16x8 pb[4];
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb) {
       float p[16];
@@ -274,7 +275,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
       constexpr int DBB = DB < 4 ? DB : 4;
 #pragma unroll
       for (int d0 = 0; d0 < DB; d0 += DBB) {
-        bf16x8 va[DBB];
+        e16x8 va[DBB];
 #pragma unroll
         for (int db = 0; db < DBB; ++db) va[db] = tra.template read<Vt>(kk, d0 + db);
 #pragma unroll
@@ -336,15 +337,15 @@ __global__ __launch_bounds__(64 * NW) void fwd_bf16_kernel(const FwdArgs a, cons
   if (rowok) {
     if (a.lse != nullptr && hh == 0)
       a.lse[((int64_t)b * a.H + h) * a.Sq + i] = has ? m * a.scale + __logf(l) : 0.f;
-    bf16_t *optr = reinterpret_cast<bf16_t *>(a.o) + b * a.o_sb + (int64_t)i * a.o_ss + h * a.o_sh;
+    e16_t *optr = reinterpret_cast<e16_t *>(a.o) + b * a.o_sb + (int64_t)i * a.o_ss + h * a.o_sh;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
-        bf16x4 w;
+        e16x4 w;
 #pragma unroll
-        for (int x = 0; x < 4; ++x) w[x] = (bf16_t)(o[db][4 * r4 + x] * inv);
-        *reinterpret_cast<bf16x4 *>(optr + 32 * db + 8 * r4 + 4 * hh) = w;
+        for (int x = 0; x < 4; ++x) w[x] = (e16_t)(o[db][4 * r4 + x] * inv);
+        *reinterpret_cast<e16x4 *>(optr + 32 * db + 8 * r4 + 4 * hh) = w;
       }
   }
 }
@@ -413,11 +414,11 @@ __global__ __launch_bounds__(256) void fwd_combine_kernel(const FwdArgs a, const
   }
   const bool has = lsum > 0.f;
   const float inv = has ? 1.f / lsum : 0.f;
-  bf16x4 w;
+  e16x4 w;
 #pragma unroll
-  for (int x = 0; x < 4; ++x) w[x] = (bf16_t)(acc[x] * inv);
-  bf16_t *optr = reinterpret_cast<bf16_t *>(a.o) + b * a.o_sb + (int64_t)i * a.o_ss + h * a.o_sh;
-  *reinterpret_cast<bf16x4 *>(optr + 32 * db + 8 * r4 + 4 * hh) = w;
+  for (int x = 0; x < 4; ++x) w[x] = (e16_t)(acc[x] * inv);
+  e16_t *optr = reinterpret_cast<e16_t *>(a.o) + b * a.o_sb + (int64_t)i * a.o_ss + h * a.o_sh;
+  *reinterpret_cast<e16x4 *>(optr + 32 * db + 8 * r4 + 4 * hh) = w;
   if (a.lse != nullptr && db == 0 && r4 == 0 && hh == 0)
     a.lse[((int64_t)b * a.H + h) * a.Sq + i] = has ? mx * a.scale + __logf(lsum) : 0.f;
 }
@@ -426,13 +427,13 @@ __global__ __launch_bounds__(256) void fwd_combine_kernel(const FwdArgs a, const
 template <int D, int NW, bool SPLIT, bool TWOSEG>
 static int launch_fwd_seg(const FwdArgs &a, const SplitArgs &sp, hipStream_t st) {
   constexpr size_t stages = fwd_stage_bytes<D, SPLIT>();
-  if (!allow_dynamic_lds<&fwd_bf16_kernel<D, NW, SPLIT, TWOSEG>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
+  if (!allow_dynamic_lds<&fwd_mfma_kernel<D, NW, SPLIT, TWOSEG>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
   const int tiles = (a.Sk0 + 63) / 64 + (a.Sk - a.Sk0 + 63) / 64;
   if (!SPLIT && !needed_table_fits(stages, tiles)) return BCATTN_ERR_UNSUPPORTED;
   const size_t smem = stages + (SPLIT ? 0 : needed_table_bytes(tiles));
   const int R = a.G * a.Sq;
   const int ntile_r = (R + 32 * NW - 1) / (32 * NW);
-  hipLaunchKernelGGL((fwd_bf16_kernel<D, NW, SPLIT, TWOSEG>),
+  hipLaunchKernelGGL((fwd_mfma_kernel<D, NW, SPLIT, TWOSEG>),
                      dim3(xcd_grid((unsigned)(ntile_r * (SPLIT ? sp.nsplit : 1) * a.Hkv * a.B))), dim3(64 * NW),
                      smem, st, a, sp);
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
@@ -443,7 +444,7 @@ static int launch_fwd_t(const FwdArgs &a, const SplitArgs &sp, hipStream_t st) {
   return a.Sk > a.Sk0 ? launch_fwd_seg<D, NW, SPLIT, true>(a, sp, st) : launch_fwd_seg<D, NW, SPLIT, false>(a, sp, st);
 }
 
-int launch_fwd_bf16(const FwdArgs &a, int D, hipStream_t st) {
+int launch_fwd_mfma(const FwdArgs &a, int D, hipStream_t st) {
   const int R = a.G * a.Sq;
   const SplitArgs sp{nullptr, nullptr, 1, 0};
   switch (D) {
@@ -492,11 +493,11 @@ static int launch_split(const FwdArgs &a, const SplitArgs &sp, hipStream_t st) {
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
 }
 
-int launch_fwd_kvcache_bf16(const FwdArgs &a, const SplitArgs &sp_in, int D, hipStream_t st) {
+int launch_fwd_kvcache_mfma(const FwdArgs &a, const SplitArgs &sp_in, int D, hipStream_t st) {
   SplitArgs sp = sp_in;
   int ns, tps;
   plan_split(a.B, a.Sq, a.Sk0, a.Sk, a.H, a.Hkv, &ns, &tps);
-  if (ns <= 1) return launch_fwd_bf16(a, D, st);
+  if (ns <= 1) return launch_fwd_mfma(a, D, st);
   sp.nsplit = ns;
   sp.tiles_per_split = tps;
   switch (D) {
@@ -511,4 +512,5 @@ int launch_fwd_kvcache_bf16(const FwdArgs &a, const SplitArgs &sp_in, int D, hip
   }
 }
 
+}  // namespace BCATTN_ELEM_NS
 }  // namespace bcattn

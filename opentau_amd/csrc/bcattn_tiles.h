@@ -7,6 +7,7 @@
 #include "bcattn_common.h"
 
 namespace bcattn {
+inline namespace BCATTN_ELEM_NS {
 
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -172,7 +173,7 @@ __device__ __forceinline__ int opaque_add(int x, int c) {
   asm("v_add_u32 %0, %1, %2" : "=v"(r) : "s"(c), "v"(x));
   return r;
 }
-typedef const __attribute__((address_space(3))) bf16x8 lds_bf16x8_t;
+typedef const __attribute__((address_space(3))) e16x8 lds_e16x8_t;
 
 // Row operand of a 32x32x16 product: row (rbase + lane%32), columns
 // 16*ks + 8*(lane/32) .. +7.  rbase must be a multiple of 16 rows.
@@ -191,11 +192,11 @@ struct RowAddr {
   }
   // T0: byte offset of the tile in the tile area
   template <int T0>
-  __device__ __forceinline__ bf16x8 read(int rbase, int ks) const {
+  __device__ __forceinline__ e16x8 read(int rbase, int ks) const {
     constexpr int A = T0 / anchor_spacing<D>();
     static_assert(A < kMaxAnchors, "tile beyond the last anchor");
     const int addr = a[A][ks] + (T0 - A * anchor_spacing<D>()) + rbase * Tile<D>::kRowBytes;
-    return *reinterpret_cast<lds_bf16x8_t *>(static_cast<uintptr_t>((uint32_t)addr));
+    return *reinterpret_cast<lds_e16x8_t *>(static_cast<uintptr_t>((uint32_t)addr));
   }
 };
 
@@ -227,7 +228,7 @@ struct TrAddr {
     }
   }
   template <int T0>
-  __device__ __forceinline__ bf16x8 read(int kk, int db) const {
+  __device__ __forceinline__ e16x8 read(int kk, int db) const {
     constexpr int A = T0 / anchor_spacing<D>();
     static_assert(A < kMaxAnchors, "tile beyond the last anchor");
     return read_from<A>((T0 - A * anchor_spacing<D>()) + 16 * kk * Tile<D>::kRowBytes, db);
@@ -235,14 +236,14 @@ struct TrAddr {
   // The same with a tile offset known only at run time (costs an add per read): `off`
   // is in bytes from anchor A.
   template <int A>
-  __device__ __forceinline__ bf16x8 read_from(int off, int db) const {
+  __device__ __forceinline__ e16x8 read_from(int off, int db) const {
     const s16x4 l =
         __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t *)static_cast<uintptr_t>((uint32_t)(lo[A][db] + off)));
     const s16x4 h =
         __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t *)static_cast<uintptr_t>((uint32_t)(hi[A][db] + off)));
     typedef short s16x8 __attribute__((ext_vector_type(8)));
     const s16x8 both = __builtin_shufflevector(l, h, 0, 1, 2, 3, 4, 5, 6, 7);
-    return __builtin_bit_cast(bf16x8, both);
+    return __builtin_bit_cast(e16x8, both);
   }
 };
 
@@ -439,4 +440,5 @@ __device__ __forceinline__ void tile_burst(int first, int end, Issue issue, Comp
   }
 }
 
+}  // namespace BCATTN_ELEM_NS
 }  // namespace bcattn

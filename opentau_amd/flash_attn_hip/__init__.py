@@ -83,7 +83,8 @@ def make_att_block_ids(
 # --------------------------------------------------------------------------- #
 # raw calls through the C ABI
 # --------------------------------------------------------------------------- #
-_DTYPES = {torch.float32: (_loader.DTYPE_F32, 4), torch.bfloat16: (_loader.DTYPE_BF16, 8)}
+_DTYPES = {torch.float32: (_loader.DTYPE_F32, 4), torch.bfloat16: (_loader.DTYPE_BF16, 8),
+           torch.float16: (_loader.DTYPE_F16, 8)}
 
 
 def _operand(t: torch.Tensor, vec: int) -> torch.Tensor:
@@ -122,7 +123,7 @@ def _check_inputs(q, k, v):
     if not q.is_cuda:
         raise RuntimeError("flash_hip attention needs tensors on a HIP device; there is no CPU fallback")
     if q.dtype not in _DTYPES:
-        raise RuntimeError(f"flash_hip attention supports float32 and bfloat16, got {q.dtype}")
+        raise RuntimeError(f"flash_hip attention supports float32, bfloat16 and float16, got {q.dtype}")
     if k.dtype != q.dtype or v.dtype != q.dtype:
         raise RuntimeError("q, k and v must share one dtype")
     if q.ndim != 4 or k.ndim != 4 or v.ndim != 4:

@@ -21,7 +21,7 @@ ABI_VERSION = 1
 
 # status codes of include/bcattn.h
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_LAUNCH = 0, -1, -2, -3, -4
-DTYPE_F32, DTYPE_BF16 = 0, 1
+DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
 BWD_DELTA, BWD_DQ, BWD_DKV = 1, 2, 4
 
 EXPORTS = (

@@ -196,6 +196,61 @@ def test_large_group_kernels_head_dim_128(pattern, sq, cross, pad_mid):
         assert rel_l2(got, ref) <= 1e-2, name
 
 
+# --------------------------------------------------------------------------- #
+# float16: the reference's kernel tests run each case in float16 and bfloat16
+# (tests/policies/test_flash_attn_cuda.py:204, :239, :283, :306) with tolerance 1e-2 for float16
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("pattern", PATTERNS)
+@pytest.mark.parametrize("head_dim", [64, 128, 256])
+def test_fp16_forward_and_backward_match_reference(pattern, head_dim):
+    b, sq, h, hkv = 2, 70, 4, 2
+    ids = make_blocks(b, sq, pattern, pad_tail=5)
+    q, k, v = _qkv(b, sq, sq, h, hkv, head_dim, torch.float16)
+    go = randn((b, sq, h, head_dim), torch.float16, 9)
+    scale = head_dim**-0.5
+    out, dq, dk, dv = _fwd_bwd(q, k, v, go, ids, scale)
+    assert out.dtype == dq.dtype == dk.dtype == dv.dtype == torch.float16
+    qm = ids[2][:, :, None, None]
+    ref = eager.eager_from_block_ids(q, k, v, *ids, scale).float()  # float16 P.V, the reference's cast order
+    torch.testing.assert_close(out.float() * qm, ref * qm, atol=1e-2, rtol=1e-2)
+    assert rel_l2(out.float() * qm, ref * qm) <= 2e-3
+    _, rq, rk, rv = eager.eager_grads(q.float(), k.float(), v.float(), go.float(), *ids, scale)
+    for got, want, name in ((dq.float() * qm, rq * qm, "dq"), (dk.float(), rk, "dk"), (dv.float(), rv, "dv")):
+        torch.testing.assert_close(got, want, atol=1e-2, rtol=1e-2)
+        assert rel_l2(got, want) <= 2e-3, name
+
+
+@pytest.mark.parametrize("sq,cross,pad_mid", [(300, 0, None), (257, 0, (40, 200)), (129, 190, None)])
+def test_fp16_large_group_kernels_head_dim_128(sq, cross, pad_mid):
+    b, h, hkv, d = 2, 8, 1, 128
+    ids = make_blocks(b, sq, "prefixlm", cross=cross, pad_tail=0 if cross else 9, pad_mid=pad_mid)
+    q, k, v = _qkv(b, sq, cross + sq, h, hkv, d, torch.float16, seed=11)
+    go = randn((b, sq, h, d), torch.float16, 19)
+    scale = d**-0.5
+    out, dq, dk, dv = _fwd_bwd(q, k, v, go, ids, scale)
+    ro, rq, rk, rv = eager.eager_grads(q.float(), k.float(), v.float(), go.float(), *ids, scale)
+    qm = ids[2][:, :, None, None]
+    assert rel_l2(out.float() * qm, ro * qm) <= 2e-3
+    for got, want, name in ((dq.float() * qm, rq * qm, "dq"), (dk.float(), rk, "dk"), (dv.float(), rv, "dv")):
+        torch.testing.assert_close(got, want, atol=1e-2, rtol=1e-2)
+        assert rel_l2(got, want) <= 2e-3, name
+
+
+def test_fp16_kvcache_equals_concat():
+    b, sq, h, hkv, d, cross = 2, 50, 8, 1, 256, 968
+    ids = make_blocks(b, sq, "prefixlm", cross=cross)
+    q, k, v = _qkv(b, sq, cross + sq, h, hkv, d, torch.float16, seed=3)
+    scale = d**-0.5
+    gi = [g(t) for t in ids]
+    whole, _ = fa.forward_raw(g(q), g(k), g(v), *gi, scale)
+    split = fa.flash_attn_blockmask_kvcache(g(q), g(k[:, :cross]), g(v[:, :cross]), g(k[:, cross:]), g(v[:, cross:]),
+                                            *gi, scale)
+    assert split.dtype == torch.float16
+    assert rel_l2(split.float().cpu(), whole.float().cpu()) <= 1e-3
+    ref = eager.eager_from_block_ids(q, k, v, *ids, scale).float()
+    assert rel_l2(split.float().cpu(), ref) <= 2e-3
+
+
 def test_backward_is_bit_repeatable():
     b, sq, h, hkv, d = 2, 300, 8, 2, 128
     ids = make_blocks(b, sq, "multiblock", pad_tail=17)
@@ -317,8 +372,8 @@ def test_errors_are_raised_not_swallowed():
         fa.forward_raw(q, k, k, *ids, 0.1)
     with pytest.raises(RuntimeError, match="dtype"):
         fa.forward_raw(k, k.float(), k, *ids, 0.1)
-    with pytest.raises(RuntimeError, match="float32 and bfloat16"):
-        fa.forward_raw(k.half(), k.half(), k.half(), *ids, 0.1)
+    with pytest.raises(RuntimeError, match="float32, bfloat16 and float16"):
+        fa.forward_raw(k.double(), k.double(), k.double(), *ids, 0.1)
     with pytest.raises(RuntimeError, match="block ids"):
         fa.forward_raw(k, k, k, ids[0][:, :4], ids[1], ids[2][:, :4], ids[3], 0.1)
     with pytest.raises(RuntimeError, match="CPU"):
