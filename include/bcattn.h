@@ -11,8 +11,8 @@
  * torch types, no device allocation: the caller owns every buffer (outputs and
  * the workspace), no pointer is retained after return, and every call is
  * asynchronous with respect to the host on the stream it is given.  The one
- * thing the library keeps is a helper stream and two events per device, made
- * on the first bcattn_bwd call that computes all gradients: its two large
+ * thing the library keeps is a helper stream and two events per device (and
+ * 16-bit element type), made on the first bcattn_bwd call that computes all gradients: its two large
  * kernels run side by side, forked from and joined to the given stream, so
  * work enqueued on that stream afterwards still sees all of the call's results
  * (BCATTN_SERIAL_BACKWARD=1 in the environment keeps everything on the given
