@@ -130,6 +130,23 @@ def _check_inputs(q, k, v):
         raise RuntimeError("q, k, v must be (B, S, H, D)")
 
 
+_MFMA_HEAD_DIMS = (64, 128, 256)
+
+
+def _head_dim_padding(q: torch.Tensor) -> int:
+    """Zero columns to append so that a 16-bit head_dim the reference accepts (any multiple of 32
+    up to 256, ``flash_blockmask.cu:1141``) reaches one the MFMA kernels are built for.  Zero
+    columns change no dot product and yield zero output / gradient columns, which are dropped."""
+    d = q.shape[-1]
+    if q.dtype == torch.float32 or d in _MFMA_HEAD_DIMS or d % 32 or not 0 < d <= 256:
+        return 0
+    return next(m for m in _MFMA_HEAD_DIMS if m > d) - d
+
+
+def _padded(t: torch.Tensor | None, n: int) -> torch.Tensor | None:
+    return None if t is None else torch.nn.functional.pad(t, (0, n))
+
+
 def forward_raw(
     q,
     k,
@@ -156,6 +173,13 @@ def forward_raw(
     """
     lib = _loader.require_library()
     _check_inputs(q, k, v)
+    extra = _head_dim_padding(q)
+    if extra:
+        o, lse = forward_raw(_padded(q, extra), _padded(k, extra), _padded(v, extra), q_blk, k_blk, q_valid, k_valid,
+                             scale, _padded(k_new, extra), _padded(v_new, extra), kvcache=kvcache,
+                             workspace=workspace, summary_ready=summary_ready, want_lse=want_lse)
+        o = o[..., : q.shape[-1]]
+        return (o.contiguous() if out is None else out.copy_(o)), lse
     code, vec = _DTYPES[q.dtype]
     b, sq, h, d = q.shape
     sk0, hkv = k.shape[1], k.shape[2]
@@ -203,6 +227,15 @@ def backward_raw(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale
     """
     lib = _loader.require_library()
     _check_inputs(q, k, v)
+    extra = _head_dim_padding(q)
+    if extra:
+        d = q.shape[-1]
+        got = backward_raw(*(_padded(t, extra) for t in (d_out, q, k, v, out)), lse, q_blk, k_blk, q_valid, k_valid,
+                           scale, stages=stages, workspace=workspace, summary_ready=summary_ready)
+        got = tuple(t[..., :d] for t in got)
+        if grads is not None:
+            return tuple(dst.copy_(src) for dst, src in zip(grads, got))
+        return tuple(t.contiguous() for t in got)
     code, vec = _DTYPES[q.dtype]
     b, sq, h, d = q.shape
     sk, hkv = k.shape[1], k.shape[2]

@@ -251,6 +251,26 @@ def test_fp16_kvcache_equals_concat():
     assert rel_l2(split.float().cpu(), ref) <= 2e-3
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("head_dim", [32, 96, 160, 224])
+def test_other_head_dims_the_reference_accepts(dtype, head_dim):
+    """The reference takes any head_dim that is a multiple of 32 up to 256
+    (``flash_blockmask.cu:1141``); those without a kernel of their own run zero-padded through the
+    next larger one."""
+    b, sq, h, hkv = 2, 70, 4, 2
+    ids = make_blocks(b, sq, "multiblock", pad_tail=5)
+    q, k, v = _qkv(b, sq, sq, h, hkv, head_dim, dtype)
+    go = randn((b, sq, h, head_dim), dtype, 9)
+    scale = head_dim**-0.5
+    out, dq, dk, dv = _fwd_bwd(q, k, v, go, ids, scale)
+    assert out.shape == q.shape and dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
+    ro, rq, rk, rv = eager.eager_grads(q.float(), k.float(), v.float(), go.float(), *ids, scale)
+    qm = ids[2][:, :, None, None]
+    for got, want, name in ((out.float() * qm, ro * qm, "out"), (dq.float() * qm, rq * qm, "dq"),
+                            (dk.float(), rk, "dk"), (dv.float(), rv, "dv")):
+        assert rel_l2(got, want) <= 1e-2, name
+
+
 def test_backward_is_bit_repeatable():
     b, sq, h, hkv, d = 2, 300, 8, 2, 128
     ids = make_blocks(b, sq, "multiblock", pad_tail=17)
