@@ -1,7 +1,7 @@
 // Block-causal attention backward, bf16 in / fp32 accumulate, gfx950 MFMA.
 //
 // Three kernels, no atomics, so gradients are bit-repeatable:
-//   prep    delta[b,h,i] = sum_d O*dO, and log2e*LSE (+inf on rows that take no
+//   prep    delta[b,h,i] = sum_d O*dO (stored negated), and log2e*LSE (+inf on rows that take no
 //           part), both padded to whole 64-row tiles so that the dK/dV kernel can
 //           pull them into LDS with one buffer load
 //   dQ      a workgroup owns 32*NW packed query rows and streams key tiles;
@@ -56,7 +56,7 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const BwdArgs a) {
   for (int o = LPR / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
   if (row < total && c == 0) {
     const bool ok = real && a.q_valid[(int64_t)b * a.Sq + i] != 0;
-    a.delta[row] = ok ? acc : 0.f;
+    a.delta[row] = ok ? -acc : 0.f;  // stored negated: the dK/dV pairs start their dP accumulators from it
     a.lse2[row] = ok ? a.lse[((int64_t)b * a.H + h) * a.Sq + i] * kLog2e : INFINITY;
   }
 }
@@ -115,7 +115,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   }
   const int64_t stat = ((int64_t)b * a.H + h) * a.Sq_pad + i;
   const float lse2 = rowok ? a.lse2[stat] : INFINITY;  // +inf on rows that take no part
-  const float delta = rowok ? a.delta[stat] : 0.f;
+  const float ndelta = rowok ? a.delta[stat] : 0.f;  // -delta
 
   const int qmax_w = wave_max_i(qv ? qb : kIntMin);
   const int qmin_w = wave_min_i(qv ? qb : kIntMax);
@@ -225,7 +225,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
         for (int x = 0; x < 4; ++x) {
           float p = fast_exp2(s[4 * r4 + x] * c - lse2);
           if (MASKED && kb4[x] > qb) p = 0.f;
-          ds[4 * r4 + x] = p * (dp[4 * r4 + x] - delta);
+          ds[4 * r4 + x] = p * (dp[4 * r4 + x] + ndelta);
         }
       }
       e16x8 dsb[2];
@@ -467,7 +467,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
             float pv = fast_exp2(s[mb][4 * r4 + x] * c - lse4[x]);
             if (MASKED && kb > qb4[x]) pv = 0.f;
             p[4 * r2 + x] = pv;
-            if (WANT_DK) ds[4 * r2 + x] = pv * (dp[mb][4 * r4 + x] - del4[x]);
+            if (WANT_DK) ds[4 * r2 + x] = pv * (dp[mb][4 * r4 + x] + del4[x]);  // del4 holds -delta
           }
         }
         if (WANT_DV) pb[mb][half] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
@@ -847,6 +847,18 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
     f32x16 dp;
 #pragma unroll
     for (int x = 0; x < 16; ++x) dp[x] = 0.f;
+    if constexpr (CUR) {
+      // the chain of products starts from -delta of the half's queries (one value per
+      // accumulator register, the same in every lane of a half wave): dP - delta costs no
+      // vector instruction
+      constexpr int NDEL = CS * (3 * 256) + 256;
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const f32x4 nd4 = lds_f32x4(aux_lane + NDEL + (32 * mb + 8 * r4) * 4);
+#pragma unroll
+        for (int x = 0; x < 4; ++x) dp[4 * r4 + x] = nd4[x];
+      }
+    }
     if constexpr (CUR)
       static_for<DK>([&](auto i_c) {
         constexpr int i = decltype(i_c)::value;
@@ -856,24 +868,18 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
     else
       static_for<LPT>([&](auto part) { bg(part); });
     if constexpr (PREV) {
-      constexpr int AUX = PS * (3 * 256) + 256;  // delta of the previous half's stage
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         const e16x8 pb = lds_e16x8(x_lane + (1 - xcur) * XBYTES + half * 1024);
         float ds[8];
 #pragma unroll
-        for (int r2 = 0; r2 < 2; ++r2) {
-          const int r4 = 2 * half + r2;
-          const f32x4 del4 = lds_f32x4(aux_lane + AUX + (32 * pmb + 8 * r4) * 4);
-#pragma unroll
-          for (int x = 0; x < 4; ++x) ds[4 * r2 + x] = (float)pb[4 * r2 + x] * (dp_prev[4 * r4 + x] - del4[x]);
-        }
+        for (int x = 0; x < 8; ++x) ds[x] = (float)pb[x] * dp_prev[8 * half + x];  // dp_prev = dP - delta
         dsb[half] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
       }
     }
     if constexpr (CUR) {
       // per product of dP: its row read and a share of the dS arithmetic
-      constexpr int VA = PREV ? (4 * 16 + DK - 1) / DK : 0;
+      constexpr int VA = PREV ? (3 * 16 + DK - 1) / DK : 0;
       __builtin_amdgcn_sched_group_barrier(0x100, (PREV ? 6 : 0) + 4, 0);
 #pragma unroll
       for (int x = 0; x < DK; ++x) {
@@ -912,19 +918,13 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
                            acc[i % DB]);
   };
   auto ds_last = [&](int stage) __attribute__((always_inline)) {
-    const int aux_stage = aux_lane + stage * (3 * 256) + 256;  // delta of the last tile's stage
     e16x8 dsb[2];
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const e16x8 pb = lds_e16x8(x_lane + XBYTES + half * 1024);  // the last half is an odd one
       float ds[8];
 #pragma unroll
-      for (int r2 = 0; r2 < 2; ++r2) {
-        const int r4 = 2 * half + r2;
-        const f32x4 del4 = lds_f32x4(aux_stage + (32 + 8 * r4) * 4);
-#pragma unroll
-        for (int x = 0; x < 4; ++x) ds[4 * r2 + x] = (float)pb[4 * r2 + x] * (dp_prev[4 * r4 + x] - del4[x]);
-      }
+      for (int x = 0; x < 8; ++x) ds[x] = (float)pb[x] * dp_prev[8 * half + x];
       dsb[half] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
     }
     constexpr int A = L::tile(0, 0) / anchor_spacing<D>();

@@ -143,7 +143,7 @@ struct BwdArgs {
   void *dq, *dk, *dv;
   int64_t dq_sb, dq_ss, dq_sh, dk_sb, dk_ss, dk_sh, dv_sb, dv_ss, dv_sh;
   const float *lse;
-  float *delta;  // (B,H,Sq_pad): row sums of O*dO, 0 on rows that take no part
+  float *delta;  // (B,H,Sq_pad): minus the row sums of O*dO, 0 on rows that take no part
   float *lse2;   // (B,H,Sq_pad): log2e*LSE, +inf on rows that take no part
   const int32_t *q_blk, *k_blk;
   const uint8_t *q_valid, *k_valid;
