@@ -187,7 +187,8 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int x = 0; x < 16; ++x) o[db][x] = 0.f;
-  float m = -INFINITY;  // running max of the raw (unscaled) scores
+  float m = -INFINITY;  // reference point of the row's exponentials, in raw (unscaled) scores
+  float moff = 0.f;     // the same times scale*log2e (0 while there is none)
   float l = 0.f;        // this lane half's share of the running sum
   const float c = a.scale * kLog2e;
 
@@ -234,41 +235,62 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
             if (kb4[x] > qb) s[mb][4 * r4 + x] = -INFINITY;
         }
     }
-    float mloc = s[0][0];
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-      for (int x = 0; x < 16; ++x) mloc = fmaxf(mloc, s[mb][x]);
-    mloc = fmaxf(mloc, swap32(mloc));
-    // The reference point of the exponentials follows the row maximum only when that has
-    // grown by more than 2^8 (in the exponent): a stale reference leaves P <= 256, which
-    // bf16 and the fp32 sums hold as well as P <= 1, and the accumulators are rescaled
-    // on a few tiles per row instead of on nearly every one.  O / l and the log-sum-exp
-    // do not depend on the reference.
-    const bool grow = (mloc - m) * c > 8.f;  // false for a fully masked tile (mloc = -inf)
-    const float mnew = grow ? mloc : m;
-    const float moff = (mnew == -INFINITY) ? 0.f : mnew * c;
-    if (__any(grow)) {
-      const float corr = fast_exp2(m * c - moff);
-      l *= corr;
-#pragma unroll
-      for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int x = 0; x < 16; ++x) o[db][x] *= corr;
-    }
-    m = mnew;
+    // The exponentials are taken against the reference point the row already has, and the tile's
+    // share of the row sum tells whether that was good enough: every P is at most the sum, so a
+    // sum of at most 2^13 means no P left the range that bf16 / fp16 and the fp32 sums hold as
+    // well as P <= 1.  Only when a row's sum is larger (or not a number), or a valid row has no
+    // reference yet, does the wave find the row maxima, move the references that have been
+    // outgrown by more than 2^8 and take the tile's exponentials again.  O / l and the
+    // log-sum-exp do not depend on the reference, and almost every tile skips the maximum.
+    constexpr float kSumMax = 8192.f;
     e16x8 pb[4];
+    float lt = 0.f;
+    auto exponentials = [&]() __attribute__((always_inline)) {
+      lt = 0.f;
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb) {
-      float p[16];
+      for (int mb = 0; mb < 2; ++mb) {
+        float p[16];
 #pragma unroll
-      for (int x = 0; x < 16; ++x) {
-        p[x] = fast_exp2(s[mb][x] * c - moff);
-        l += p[x];
+        for (int x = 0; x < 16; ++x) {
+          p[x] = fast_exp2(s[mb][x] * c - moff);
+          lt += p[x];
+        }
+        pb[2 * mb] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
+        pb[2 * mb + 1] = pack8(p[8], p[9], p[10], p[11], p[12], p[13], p[14], p[15]);
       }
-      pb[2 * mb] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
-      pb[2 * mb + 1] = pack8(p[8], p[9], p[10], p[11], p[12], p[13], p[14], p[15]);
+    };
+    // (At head_dim 256, one wave per SIMD and a full register file, the second pass costs more
+    // than the maximum it saves: there the maxima are found on every tile.)
+    constexpr bool kCheckBySum = D <= 128;
+    bool again = true;
+    if constexpr (kCheckBySum) {
+      exponentials();
+      again = qv && (!(lt <= kSumMax) || m == -INFINITY);
     }
+    if (!kCheckBySum || __any(again)) {
+      float mloc = s[0][0];
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int x = 0; x < 16; ++x) mloc = fmaxf(mloc, s[mb][x]);
+      mloc = fmaxf(mloc, swap32(mloc));
+      const bool grow = (mloc - m) * c > 8.f;  // false for a fully masked tile (mloc = -inf)
+      const float mnew = grow ? mloc : m;
+      const float moff_new = (mnew == -INFINITY) ? 0.f : mnew * c;
+      if (__any(grow)) {
+        // 1 where the reference stays; a row without one has accumulated nothing that counts
+        const float corr = (m == -INFINITY) ? 0.f : fast_exp2(moff - moff_new);
+        l *= corr;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int x = 0; x < 16; ++x) o[db][x] *= corr;
+      }
+      m = mnew;
+      moff = moff_new;
+      exponentials();
+    }
+    l += lt;
     // O^T += V^T P^T: the DB accumulators are independent, so the key steps run outermost.
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
@@ -344,7 +366,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
       for (int r4 = 0; r4 < 4; ++r4) {
         e16x4 w;
 #pragma unroll
-        for (int x = 0; x < 4; ++x) w[x] = (e16_t)(o[db][4 * r4 + x] * inv);
+        for (int x = 0; x < 4; ++x) w[x] = has ? (e16_t)(o[db][4 * r4 + x] * inv) : (e16_t)0.f;
         *reinterpret_cast<e16x4 *>(optr + 32 * db + 8 * r4 + 4 * hh) = w;
       }
   }

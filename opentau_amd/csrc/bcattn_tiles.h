@@ -179,12 +179,15 @@ typedef const __attribute__((address_space(3))) e16x8 lds_e16x8_t;
 // 16*ks + 8*(lane/32) .. +7.  rbase must be a multiple of 16 rows.
 template <int D>
 struct RowAddr {
-  int a[kMaxAnchors][D / 16];
+  // The swizzle permutes the 16 slots of each 256 bytes of a row among themselves, so steps
+  // 8 apart (256 bytes apart in the row) share a lane address and differ by an immediate.
+  static constexpr int kDistinct = D / 16 < 8 ? D / 16 : 8;
+  int a[kMaxAnchors][kDistinct];
   // lds0: LDS byte address of the tile area
   __device__ __forceinline__ void init(int lane, uint32_t lds0) {
     const int n = lane & 31, hh = lane >> 5;
 #pragma unroll
-    for (int ks = 0; ks < D / 16; ++ks) {
+    for (int ks = 0; ks < kDistinct; ++ks) {
       a[0][ks] = (int)lds0 + Tile<D>::off(n, 2 * ks + hh);
 #pragma unroll
       for (int i = 1; i < kMaxAnchors; ++i) a[i][ks] = opaque_add(a[0][ks], i * anchor_spacing<D>());
@@ -195,7 +198,8 @@ struct RowAddr {
   __device__ __forceinline__ e16x8 read(int rbase, int ks) const {
     constexpr int A = T0 / anchor_spacing<D>();
     static_assert(A < kMaxAnchors, "tile beyond the last anchor");
-    const int addr = a[A][ks] + (T0 - A * anchor_spacing<D>()) + rbase * Tile<D>::kRowBytes;
+    const int addr =
+        a[A][ks % kDistinct] + (T0 - A * anchor_spacing<D>()) + rbase * Tile<D>::kRowBytes + (ks / kDistinct) * 256;
     return *reinterpret_cast<lds_e16x8_t *>(static_cast<uintptr_t>((uint32_t)addr));
   }
 };
@@ -210,14 +214,16 @@ struct RowAddr {
 // columns 32*db + 16*(group%2) + 4*(i%4) .. +3.
 template <int D>
 struct TrAddr {
-  int lo[kMaxAnchors][D / 32], hi[kMaxAnchors][D / 32];
+  // (head_dim blocks 4 apart are 256 bytes apart in the row: same lane address, other immediate)
+  static constexpr int kDistinct = D / 32 < 4 ? D / 32 : 4;
+  int lo[kMaxAnchors][kDistinct], hi[kMaxAnchors][kDistinct];
   __device__ __forceinline__ void init(int lane, uint32_t lds0) {
     const int i = lane & 15, grp = (lane >> 4) & 1, hh = lane >> 5;
     const int row = 4 * hh + (i >> 2);
     const int slot = 2 * grp + ((i & 3) >> 1);
     const int byte = 8 * (i & 1);
 #pragma unroll
-    for (int db = 0; db < D / 32; ++db) {
+    for (int db = 0; db < kDistinct; ++db) {
       lo[0][db] = (int)lds0 + Tile<D>::off(row, 4 * db + slot) + byte;
       hi[0][db] = (int)lds0 + Tile<D>::off(row + 8, 4 * db + slot) + byte;
 #pragma unroll
@@ -237,10 +243,11 @@ struct TrAddr {
   // is in bytes from anchor A.
   template <int A>
   __device__ __forceinline__ e16x8 read_from(int off, int db) const {
-    const s16x4 l =
-        __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t *)static_cast<uintptr_t>((uint32_t)(lo[A][db] + off)));
-    const s16x4 h =
-        __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t *)static_cast<uintptr_t>((uint32_t)(hi[A][db] + off)));
+    const int far = (db / kDistinct) * 256;
+    const s16x4 l = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (lds_s16x4_t *)static_cast<uintptr_t>((uint32_t)(lo[A][db % kDistinct] + off + far)));
+    const s16x4 h = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (lds_s16x4_t *)static_cast<uintptr_t>((uint32_t)(hi[A][db % kDistinct] + off + far)));
     typedef short s16x8 __attribute__((ext_vector_type(8)));
     const s16x8 both = __builtin_shufflevector(l, h, 0, 1, 2, 3, 4, 5, 6, 7);
     return __builtin_bit_cast(e16x8, both);
