@@ -196,6 +196,35 @@ def test_large_group_kernels_head_dim_128(pattern, sq, cross, pad_mid):
         assert rel_l2(got, ref) <= 1e-2, name
 
 
+@pytest.mark.parametrize("head_dim", [128, 256])
+@pytest.mark.parametrize("case", ["large", "rising", "very_negative", "late_peak"])
+def test_softmax_reference_survives_extreme_scores(case, head_dim):
+    """The forward keeps a row's exponent reference until the row sums show it has been outgrown;
+    scores far outside the usual range, maxima that rise along the keys, rows whose every score is
+    hugely negative and a single late spike must all come out as the fp32 softmax does."""
+    b, sq, h, hkv = 1, 260, 4, 1
+    ids = make_blocks(b, sq, "prefixlm", pad_tail=3)
+    q, k, v = _qkv(b, sq, sq, h, hkv, head_dim, torch.bfloat16, seed=21)
+    scale = head_dim**-0.5
+    if case == "large":
+        q = q * 24
+    elif case == "rising":  # the scores of every row grow with the key index: the reference must follow
+        k = (k.float() * 0.1 + q[:, :1, :1].float() * torch.linspace(0, 6, sq).view(1, sq, 1, 1)).to(torch.bfloat16)
+    elif case == "very_negative":  # every score of a row is around -10^3
+        k = (-q[:, :, :1].float().mean(1, keepdim=True) * 40 + k.float() * 0.05).to(torch.bfloat16)
+        q = (q[:, :, :1].float().mean(1, keepdim=True) * 8 + q.float() * 0.05).to(torch.bfloat16)
+    else:  # one key near the end dominates the rows that see it
+        k = k.clone()
+        k[:, 200] = (q[:, 100, 0] * 6).to(torch.bfloat16)
+    out, lse = _fwd(q, k, v, ids, scale)
+    vr = ids[2][:, :, None, None]
+    ref = eager.eager_from_block_ids(q, k, v, *ids, scale).float()
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    assert_close_bf16(out.float() * vr, ref * vr, "out", mabs=4e-2)
+    ref_lse = eager.attention_lse(q, k, *ids, scale)
+    torch.testing.assert_close(lse * ids[2][:, None, :], ref_lse * ids[2][:, None, :], atol=2e-3, rtol=1e-4)
+
+
 # --------------------------------------------------------------------------- #
 # float16: the reference's kernel tests run each case in float16 and bfloat16
 # (tests/policies/test_flash_attn_cuda.py:204, :239, :283, :306) with tolerance 1e-2 for float16
