@@ -184,6 +184,9 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
 #pragma unroll
     for (int x = 0; x < 16; ++x) dq[db][x] = 0.f;
   const float c = a.scale * kLog2e;
+  f32x16 nd16;
+#pragma unroll
+  for (int x = 0; x < 16; ++x) nd16[x] = ndelta;
 
   // MASKED is a compile-time copy of "some pair of this tile may be masked", so that the
   // common case carries no id reads, compares or selects at all.
@@ -194,9 +197,11 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
     const int *kb_s = reinterpret_cast<const int *>(smem + L::aux(S));
     static_for<2>([&](auto mb_c) {
       constexpr int mb = decltype(mb_c)::value;
-      f32x16 s, dp;
+      // dP starts from -delta of the lane's query (a set of registers kept for the purpose is the
+      // C operand of the chain's first product), so dS = P o dP' needs no subtraction
+      f32x16 s, dp = nd16;
 #pragma unroll
-      for (int x = 0; x < 16; ++x) s[x] = 0.f, dp[x] = 0.f;
+      for (int x = 0; x < 16; ++x) s[x] = 0.f;
       constexpr int KB = 2;  // operand reads issued ahead of the products
       static_for<DK / KB>([&](auto b_c) {
         constexpr int k0 = decltype(b_c)::value * KB;
@@ -225,7 +230,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
         for (int x = 0; x < 4; ++x) {
           float p = fast_exp2(s[4 * r4 + x] * c - lse2);
           if (MASKED && kb4[x] > qb) p = 0.f;
-          ds[4 * r4 + x] = p * (dp[4 * r4 + x] + ndelta);
+          ds[4 * r4 + x] = p * dp[4 * r4 + x];
         }
       }
       e16x8 dsb[2];
