@@ -261,18 +261,10 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   settle_loads();
   tile_pipeline<NS, LPT, LPT>(0, nt, find, issue, compute);
 
-  if (rowok) {
-    e16_t *optr = reinterpret_cast<e16_t *>(a.dq) + b * a.dq_sb + (int64_t)i * a.dq_ss + h * a.dq_sh;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        e16x4 w;
-#pragma unroll
-        for (int x = 0; x < 4; ++x) w[x] = (e16_t)(dq[db][4 * r4 + x] * a.scale);
-        *reinterpret_cast<e16x4 *>(optr + 32 * db + 8 * r4 + 4 * hh) = w;
-      }
-  }
+  // every wave is past its last tile (and its last request) before the tiles become output buffers
+  __syncthreads();
+  e16_t *optr = reinterpret_cast<e16_t *>(a.dq) + b * a.dq_sb + (int64_t)i * a.dq_ss + h * a.dq_sh;
+  store_rows_whole_lines<D>(dq, a.scale, rowok ? optr : nullptr, smem + wave * kOutBytes<D>, lane);
 }
 
 template <int D>

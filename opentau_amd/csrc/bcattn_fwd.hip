@@ -359,17 +359,18 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
   if (rowok) {
     if (a.lse != nullptr && hh == 0)
       a.lse[((int64_t)b * a.H + h) * a.Sq + i] = has ? m * a.scale + __logf(l) : 0.f;
-    e16_t *optr = reinterpret_cast<e16_t *>(a.o) + b * a.o_sb + (int64_t)i * a.o_ss + h * a.o_sh;
+  }
+  // Rows without a visible key are written as zeros whatever their accumulators hold.
+  if (!has) {
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        e16x4 w;
-#pragma unroll
-        for (int x = 0; x < 4; ++x) w[x] = has ? (e16_t)(o[db][4 * r4 + x] * inv) : (e16_t)0.f;
-        *reinterpret_cast<e16x4 *>(optr + 32 * db + 8 * r4 + 4 * hh) = w;
-      }
+      for (int x = 0; x < 16; ++x) o[db][x] = 0.f;
   }
+  // every wave is past its last tile (and its last request) before the tiles become output buffers
+  __syncthreads();
+  e16_t *optr = reinterpret_cast<e16_t *>(a.o) + b * a.o_sb + (int64_t)i * a.o_ss + h * a.o_sh;
+  store_rows_whole_lines<D>(o, inv, rowok ? optr : nullptr, smem + wave * kOutBytes<D>, lane);
 }
 
 template <int D, bool SPLIT>

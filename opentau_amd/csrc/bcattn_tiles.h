@@ -254,6 +254,47 @@ struct TrAddr {
   }
 };
 
+// Output rows of a wave, from accumulators to memory in whole lines.  A lane holds, for its
+// sequence position (lane % 32), pieces of 4 head_dim values; stored directly, one instruction
+// would touch 32 rows with 16 bytes each.  Here the wave turns its 32 x D block through a
+// private piece of LDS (`buf`, kOutBytes<D>, 16-byte aligned) so that 2*D/16 consecutive lanes write one
+// whole row: every store instruction covers whole 128-byte lines.  acc[db][4*r4 + x] is the
+// value of head_dim 32*db + 8*r4 + 4*(lane/32) + x; `row` is where the lane's position goes
+// (nullptr: nowhere); values are multiplied by `mul` first.  The caller has made sure that
+// no wave still reads or fills the tiles `buf` overlays.
+template <int D>
+constexpr int kOutPitch = 2 * D + 16;  // bytes per row in LDS: 16-byte aligned, write conflicts at their minimum
+template <int D>
+constexpr int kOutBytes = 32 * kOutPitch<D> + 32 * 8;
+template <int D>
+__device__ __forceinline__ void store_rows_whole_lines(const f32x16 *acc, float mul, e16_t *row, char *buf,
+                                                       int lane) {
+  constexpr int DB = D / 32, PITCH = kOutPitch<D>;
+  const int n = lane & 31, hh = lane >> 5;
+  e16_t **rows = reinterpret_cast<e16_t **>(buf + 32 * PITCH);
+  if (hh == 0) rows[n] = row;
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+      e16x4 w;
+#pragma unroll
+      for (int x = 0; x < 4; ++x) w[x] = (e16_t)(acc[db][4 * r4 + x] * mul);
+      *reinterpret_cast<e16x4 *>(buf + n * PITCH + (32 * db + 8 * r4 + 4 * hh) * 2) = w;
+    }
+  // (the LDS operations of one wave take effect in program order: no barrier between the
+  // lanes' writes above and the reads of other lanes' values below)
+  constexpr int LPR = 2 * D / 16;  // lanes per row, 16 bytes each
+  constexpr int RPI = 64 / LPR;    // rows per store instruction
+#pragma unroll
+  for (int it = 0; it < 32 / RPI; ++it) {
+    const int r = it * RPI + lane / LPR, col = lane % LPR;
+    const e16x8 v = *reinterpret_cast<const e16x8 *>(buf + r * PITCH + col * 16);
+    e16_t *dst = rows[r];
+    if (dst != nullptr) *reinterpret_cast<e16x8 *>(dst + col * 8) = v;
+  }
+}
+
 // f(StageC<0>{}), ..., f(StageC<N-1>{})
 template <int N, class F>
 __device__ __forceinline__ void static_for(F f);
