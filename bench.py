@@ -32,9 +32,9 @@ PEAK_HBM_GBPS = 8000.0
 # the same counter reads for a plain 1 GiB device copy (FETCH_SIZE reads half the bytes: factor 2.0;
 # WRITE_SIZE: factor 1.0).  Other workloads have no such measurement and report null.
 HBM_TRAFFIC_BYTES = {
-    ("c5", "fwd"): int((287209.6 * 2.0 + 559482.0) * 1024),
-    ("c5", "bwd_dq"): int((438911.2 * 2.0 + 531897.0) * 1024),
-    ("c5", "bwd_dkv"): int((611929.4 * 2.0 + 70432.0) * 1024),
+    ("c5", "fwd"): int((286983.2 * 2.0 + 286134.3) * 1024),
+    ("c5", "bwd_dq"): int((438147.6 * 2.0 + 281728.0) * 1024),
+    ("c5", "bwd_dkv"): int((672022.2 * 2.0 + 70432.0) * 1024),
 }
 
 
