@@ -83,11 +83,11 @@ static int check_tensor(const char *name, const bcattn_tensor &t, int vec, bool 
   return BCATTN_OK;
 }
 
-// The MFMA kernels address a (batch, head) slab of an operand through a 32-bit
-// buffer descriptor: rows * stride * 2 bytes must stay below 2^31.
 // bf16 and fp16 run the MFMA kernels
 static bool is16(int dtype) { return dtype == BCATTN_BF16 || dtype == BCATTN_F16; }
 
+// The MFMA kernels address a (batch, head) slab of an operand through a 32-bit
+// buffer descriptor: rows * stride * 2 bytes must stay below 2^31.
 static int check_span(const char *name, const bcattn_tensor &t, int rows, int D, int dtype) {
   if (!is16(dtype) || t.ptr == nullptr) return BCATTN_OK;
   if (t.stride_s < D) return fail(BCATTN_ERR_INVALID, "%s: sequence stride smaller than head_dim", name);

@@ -1,4 +1,4 @@
-// Block-causal attention backward, bf16 in / fp32 accumulate, gfx950 MFMA.
+// Block-causal attention backward, 16-bit (bf16 or fp16) in / fp32 accumulate, gfx950 MFMA.
 //
 // Three kernels, no atomics, so gradients are bit-repeatable:
 //   prep    delta[b,h,i] = sum_d O*dO (stored negated), and log2e*LSE (+inf on rows that take no
@@ -8,13 +8,17 @@
 //           dQ^T = K^T dS^T with dS^T = P^T o (dP^T - delta), all keys x queries
 //   dK/dV   a workgroup owns 128 keys of one kv head and streams the query tiles
 //           of every query head of its group, so the sum over the GQA group
-//           happens in registers; dV^T = dO^T P, dK^T = Q^T dS (queries x keys)
+//           happens in registers; dV^T = dO^T P, dK^T = Q^T dS (queries x keys).
+//           Two forms: one wave per 32 keys does all four products (any head_dim;
+//           at 256 as two launches, dV then dK), or, at head_dim 128 and long rows,
+//           two waves per 32 keys split them and pass P through LDS
 // P is recomputed from the saved log-sum-exp: P = exp2(scale*log2e*S - log2e*LSE).
+// A call that computes dQ and dK/dV runs the two kernels side by side on two streams.
 //
 // As in the forward, the 32x32 accumulator of the first product is already the B
-// operand of the second, so P / dS never leave registers.  Streamed tiles go
-// from global memory straight into swizzled LDS tiles (no registers, no LDS
-// stores), double buffered; the operand that must be contracted over the
+// operand of the second, so P / dS never leave registers inside a wave.  Streamed tiles
+// go from global memory straight into swizzled LDS tiles (no registers, no LDS
+// stores), two or three stages deep; the operand that must be contracted over the
 // sequence axis (K^T, Q^T, dO^T) is read from the same row-major tile with the
 // transposing LDS read.
 #include <cstdlib>
@@ -414,7 +418,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   // of one 32-query half runs in the shadow of the other half's matrix products:
   //   A0 | A1 + softmax0 | C0 + softmax1 | C1
   // A(mb): S = Q K^T and dP = dO V^T of queries 32mb.. (row operands from LDS)
-  // softmax(mb): P = exp2(c S - log2e LSE), dS = P o (dP - delta), packed to bf16
+  // softmax(mb): P = exp2(c S - log2e LSE), dS = P o (dP - delta), packed to 16 bits
   // C(mb): dV^T += dO^T P, dK^T += Q^T dS (transposed operands from LDS)
   // The scheduler is given the interleaving explicitly (sched_group_barrier:
   // 0x008 matrix, 0x100 LDS read, 0x002 vector ALU); MASKED is a compile-time copy
@@ -575,7 +579,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
 // ---- dK / dV with paired waves --------------------------------------------------------
 // Two waves share 32 keys and split the work of a 32-query half tile in two equal parts:
 //   the P wave   holds the K fragments and the dV accumulators:
-//                S = Q K^T, P = exp2(c S - lse) (masked), leaves P as bf16 in an LDS
+//                S = Q K^T, P = exp2(c S - lse) (masked), leaves P (16-bit) in an LDS
 //                exchange buffer, dV^T += dO^T P
 //   the dS wave  holds the V fragments and the dK accumulators:
 //                dP = dO V^T, takes P from the buffer, dS = P o (dP - delta), dK^T += Q^T dS
@@ -598,7 +602,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   constexpr int DK = D / 16, DB = D / 32;
   constexpr int NS = 3;
   using L = StageLayout<D, NS, 3 * 256>;  // per stage: Q tile, dO tile; lse2, delta, q ids
-  constexpr int XBYTES = NP * 2048;  // one exchange buffer: per pair the P of a half tile, bf16
+  constexpr int XBYTES = NP * 2048;  // one exchange buffer: per pair the P of a half tile, 16-bit
 
   extern __shared__ __align__(1024) char smem[];
   __shared__ int red_s[NP];
@@ -752,7 +756,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
 
   // State carried from one half tile to the next: what the accumulating products of the
   // previous half still need.
-  e16x8 pend[2] = {};  // P wave: P(h-1) as bf16
+  e16x8 pend[2] = {};  // P wave: P(h-1), 16-bit
   f32x16 dp_prev = {};  // dS wave: dP(h-1)
 
   // One half tile of the P wave: S(h) (a chain of dependent products), then softmax(h)
@@ -1124,7 +1128,7 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
   if (a.stages & BCATTN_BWD_DKV) {
     if constexpr (PAIRS > 0) {
       rc = launch_dkv_pair<D, PAIRS>(a, kst);
-    } else if (SPLIT) {
+    } else if constexpr (SPLIT) {
       if (!(rc = launch_dkv<D, NWK, kModeDV>(a, kst))) rc = launch_dkv<D, NWK, kModeDK>(a, kst);
     } else {
       rc = launch_dkv<D, NWK, kModeBoth>(a, kst);

@@ -19,20 +19,16 @@ typedef _Float16 e16_t;
 #define BCATTN_ELEM_NS bf16
 typedef __bf16 e16_t;
 #endif
-typedef e16_t e16x2 __attribute__((ext_vector_type(2)));
 typedef e16_t e16x4 __attribute__((ext_vector_type(4)));
 typedef e16_t e16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kWave = 64;
 constexpr int kIntMax = 0x7fffffff;
 constexpr int kIntMin = (-0x7fffffff - 1);
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr float kLn2 = 0.6931471805599453f;
 
 // Key tiles of the summary pass are this many keys wide.
 constexpr int kSumTile = 64;

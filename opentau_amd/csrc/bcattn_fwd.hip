@@ -1,21 +1,21 @@
-// Block-causal attention forward, bf16 in / fp32 accumulate, gfx950 MFMA.
+// Block-causal attention forward, 16-bit (bf16 or fp16) in / fp32 accumulate, gfx950 MFMA.
 //
-// One workgroup = 4 waves = 128 "packed" query rows of one (batch, kv head):
+// One workgroup = NW waves (4 or 8) = 32*NW "packed" query rows of one (batch, kv head):
 // packed row r = g*Sq + i runs over the G = H/Hkv query heads that share the kv
 // head, so MQA/GQA heads reuse the same K/V tile in LDS.  A wave owns 32 rows;
-// lane l owns row l%32 (its running max / sum / block id live in scalars of the
+// lane l owns row l%32 (its softmax reference / sum / block id live in scalars of the
 // lane) and the two lane halves split the contraction index.
 //
 // Scores are computed transposed, S^T = K Q^T (keys x queries), so that the
 // softmax reduction over keys is in-lane plus one exchange with lane^32, and so
 // that the 32x32 accumulator of S^T is already laid out as the B operand of
-// O^T = V^T P^T.  K tiles sit in LDS as rows, V tiles transposed.
+// O^T = V^T P^T.  K and V tiles sit in LDS as rows (as they lie in memory); V^T is read
+// with the transposing LDS read.
 #include "bcattn_tiles.h"
 
 namespace bcattn {
 inline namespace BCATTN_ELEM_NS {
 
-//
 // SPLIT: the key tiles are divided over `nsplit` workgroups per row tile; each
 // writes its unnormalised fp32 partial (O, running max, sum) and
 // `fwd_combine_kernel` merges them.  This is what lets a handful of
@@ -31,6 +31,8 @@ struct SplitStages {
   static constexpr int value = D <= 128 ? 4 : 2;
 };
 
+// TWOSEG: the keys come as two segments (cache, then new); with one segment the tile requests
+// choose nothing at run time.
 template <int D, int NW, bool SPLIT, bool TWOSEG>
 __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, const SplitArgs sp) {
   using T = Tile<D>;

@@ -1,4 +1,4 @@
-// LDS tiles of the MFMA kernels: 64 rows x D bf16, filled by buffer loads that
+// LDS tiles of the MFMA kernels: 64 rows x D 16-bit elements, filled by buffer loads that
 // write LDS directly, read either as row operands (16-byte reads) or as
 // transposed operands (ds_read_b64_tr_b16), with one XOR swizzle that keeps both
 // kinds of read free of bank conflicts.
@@ -9,7 +9,6 @@
 namespace bcattn {
 inline namespace BCATTN_ELEM_NS {
 
-typedef __attribute__((address_space(3))) void lds_void_t;
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) s16x4 lds_s16x4_t;
 
@@ -110,26 +109,13 @@ struct TileLoad {
       voff[x] = (uint32_t)(row * row_stride_elems * 2 + L * 16);
     }
   }
-  // `tile` is the LDS byte address of the tile, `soff` the byte offset of its first row
-  // in the source.
-  __device__ __forceinline__ void issue(buf_rsrc_t rsrc, uint32_t tile, uint32_t soff, int wave) const {
-    const uint32_t base = __builtin_amdgcn_readfirstlane(tile + 1024u * (uint32_t)wave);
-    const uint32_t so = __builtin_amdgcn_readfirstlane(soff);
-    issue_from<0>(rsrc, base, so);
-  }
-  // Load X of the tile alone (the same arguments as issue()).
+  // Load X of the tile: `tile` is the LDS byte address of the tile, `soff` the byte offset of
+  // the tile's first row in the source.
   template <int X>
   __device__ __forceinline__ void issue_one(buf_rsrc_t rsrc, uint32_t tile, uint32_t soff, int wave) const {
     static_assert(X < kLoads, "load index");
     dma16<X * NT * 16>(rsrc, __builtin_amdgcn_readfirstlane(tile + 1024u * (uint32_t)wave), voff[X],
                        __builtin_amdgcn_readfirstlane(soff));
-  }
-  template <int X>
-  __device__ __forceinline__ void issue_from(buf_rsrc_t rsrc, uint32_t base, uint32_t so) const {
-    if constexpr (X < kLoads) {
-      dma16<X * NT * 16>(rsrc, base, voff[X], so);
-      issue_from<X + 1>(rsrc, base, so);
-    }
   }
 };
 
@@ -137,8 +123,6 @@ struct TileLoad {
 __device__ __forceinline__ void load_row64_dwords(buf_rsrc_t rsrc, uint32_t dst, uint32_t soff, int lane) {
   dma4(rsrc, __builtin_amdgcn_readfirstlane(dst), (uint32_t)lane * 4, __builtin_amdgcn_readfirstlane(soff));
 }
-
-__device__ __forceinline__ void wait_async_loads() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // LDS layout of a tile loop: the 2*NS tiles first, one after the other and grouped by
 // kind (tile w of stage s at (w*NS + s) tile sizes: the reads of one kind of tile then
