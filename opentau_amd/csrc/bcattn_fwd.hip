@@ -224,6 +224,16 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
           s[1] = mfma32(ka1[ks], qf[k0 + ks], s[1]);
         });
       });
+      // the row reads run ahead of the products that use them (left alone, the scheduler
+      // issues each read right in front of its product)
+      constexpr int NM = 2 * DK, kAhead = NM < 8 ? NM : 8;
+      __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+      for (int x = 0; x < NM - kAhead; ++x) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
     }
     const bool needmask = !(sm.z != 0 && sm.y <= qmin_w);
     if (needmask) {
@@ -305,6 +315,17 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
 #pragma unroll
         for (int db = 0; db < DBB; ++db) o[d0 + db] = mfma32(va[db], pb[kk], o[d0 + db]);
       }
+    }
+    {
+      // two transposing reads per product, four products' worth ahead
+      constexpr int NM = 4 * DB, kAhead = 4;
+      __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
+#pragma unroll
+      for (int x = 0; x < NM - kAhead; ++x) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
     }
     return true;
   };
