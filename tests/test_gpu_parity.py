@@ -618,6 +618,45 @@ def test_traced_graph_runs_the_same_kernels():
         assert torch.equal(a, c)
 
 
+def test_calls_replay_from_a_captured_graph():
+    """A denoise step is many small calls; a caller that captures them in a HIP graph must get,
+    on every replay, what the eager calls give for the inputs then in place (the library
+    allocates nothing and clears nothing; the backward's helper stream joins the capture through
+    its events).  Replays alternate with eager work and synchronisation."""
+    b, sq, h, hkv, d, cross = 2, 50, 8, 1, 256, 200
+    ids = [g(t) for t in make_blocks(b, sq, "prefixlm", cross=cross)]
+    sids = [g(t) for t in make_blocks(b, 1100 // 8 + 3, "prefixlm", pad_tail=7)]
+    scale = d**-0.5
+    q = g(randn((b, sq, h, d), torch.bfloat16, 1))
+    kc, vc = g(randn((b, cross, hkv, d), torch.bfloat16, 2)), g(randn((b, cross, hkv, d), torch.bfloat16, 3))
+    kn, vn = g(randn((b, sq, hkv, d), torch.bfloat16, 4)), g(randn((b, sq, hkv, d), torch.bfloat16, 5))
+    s2 = sids[0].shape[1]
+    q2, k2, v2 = (g(t) for t in _qkv(b, s2, s2, 8, 1, 128, torch.bfloat16, seed=30))  # G*Sq >= 1024: two-stream backward
+    go2 = g(randn((b, s2, 8, 128), torch.bfloat16, 37))
+
+    def work():
+        o1 = fa.flash_attn_blockmask_kvcache(q, kc, vc, kn, vn, *ids, scale)
+        o2, lse2 = fa.forward_raw(q2, k2, v2, *sids, 128**-0.5)
+        return (o1, o2, *fa.backward_raw(go2, q2, k2, v2, o2, lse2, *sids, 128**-0.5))
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):  # warm-up outside the capture (first calls set attributes, make the helper stream)
+        work()
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = work()
+    for rep in range(3):
+        for t in (q, kn, q2, go2):  # new inputs in the captured buffers
+            t.copy_(g(randn(tuple(t.shape), torch.bfloat16, 100 + rep)))
+        graph.replay()
+        torch.cuda.synchronize()
+        eager_out = work()
+        torch.cuda.synchronize()
+        for got, want in zip(captured, eager_out):
+            assert torch.equal(got, want), rep
+
+
 # --------------------------------------------------------------------------- #
 # the five benchmark configurations
 # --------------------------------------------------------------------------- #
