@@ -32,9 +32,9 @@ PEAK_HBM_GBPS = 8000.0
 # the same counter reads for a plain 1 GiB device copy (FETCH_SIZE reads half the bytes: factor 2.0;
 # WRITE_SIZE: factor 1.0).  Other workloads have no such measurement and report null.
 HBM_TRAFFIC_BYTES = {
-    ("c5", "fwd"): int((286983.2 * 2.0 + 286134.3) * 1024),
-    ("c5", "bwd_dq"): int((438147.6 * 2.0 + 281728.0) * 1024),
-    ("c5", "bwd_dkv"): int((672022.2 * 2.0 + 70432.0) * 1024),
+    ("c5", "fwd"): int((286544.8 * 2.0 + 286134.8) * 1024),
+    ("c5", "bwd_dq"): int((437374.5 * 2.0 + 281728.0) * 1024),
+    ("c5", "bwd_dkv"): int((669672.8 * 2.0 + 70432.0) * 1024),
 }
 
 
@@ -45,6 +45,7 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-denoise", action="store_true", help="skip the pi0.5 denoise leg")
+    ap.add_argument("--no-others", action="store_true", help="skip the C3 / C4 steps reported beside the headline")
     ap.add_argument("--serial", action="store_true",
                     help="keep the backward's two big kernels on one stream (for per-kernel profiles)")
     ap.add_argument("--workload", default="c5", choices=["c3", "c4", "c5"])
@@ -174,7 +175,7 @@ def main() -> int:
 
     if not args.no_denoise:
         result["denoise"] = bench_denoise(torch, fa, make_denoise_workload, dev)
-        if args.workload == "c5":
+        if args.workload == "c5" and not args.no_others:
             result["other_workloads"] = {n: bench_step_only(torch, fa, make_workload, dev, n) for n in ("c3", "c4")}
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, make_workload, args.workload)
