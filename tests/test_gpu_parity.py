@@ -755,3 +755,29 @@ def test_full_size_cosmos3_properties():
     o4 = fa.flash_attn_blockmask_kvcache(q[:, npre:], k[:, :npre], v[:, :npre], k[:, npre:], v[:, npre:],
                                          *[g(t) for t in sids], w.scale)
     assert max_abs(o4.float(), out[:, npre:].float()) <= 2**-7
+
+
+@pytest.mark.parametrize("head_dim,seq", [(128, 12000), (256, 6000)])
+def test_long_sequence_against_the_oracle_on_the_gpu(head_dim, seq):
+    """Hundreds of key tiles per row (the table of needed tiles, many rounds of the stage ring, a
+    padding hole that removes whole tiles): the oracle's eager arithmetic, run here on the GPU in
+    fp32 because its S x S temporaries are too slow for the host, is the second opinion."""
+    b, h, hkv = 1, 4, 2
+    pad = torch.ones(b, seq, dtype=torch.bool)
+    pad[:, 3000:3700] = False  # whole tiles without a valid position
+    pad[:, -37:] = False
+    att = torch.zeros(b, seq, dtype=torch.int32)
+    att[:, seq // 2 :: 997] = 1  # a bidirectional first half, then blocks of 997
+    ids = fa.make_att_block_ids(pad, att)
+    q, k, v = (g(t) for t in _qkv(b, seq, seq, h, hkv, head_dim, torch.bfloat16, seed=51))
+    go = g(randn((b, seq, h, head_dim), torch.bfloat16, 57))
+    gi = [g(t) for t in ids]
+    scale = head_dim**-0.5
+    out, lse = fa.forward_raw(q, k, v, *gi, scale)
+    dq, dk, dv = fa.backward_raw(go, q, k, v, out, lse, *gi, scale)
+    ro, rq, rk, rv = eager.eager_grads(q.float(), k.float(), v.float(), go.float(), *gi, scale)
+    qm = gi[2][:, :, None, None]
+    assert rel_l2(out.float() * qm, ro * qm) <= 1e-2
+    for got, want, name in ((dq.float() * qm, rq * qm, "dq"), (dk.float(), rk, "dk"), (dv.float(), rv, "dv")):
+        assert rel_l2(got, want) <= 1e-2, name
+
