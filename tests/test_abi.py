@@ -136,3 +136,23 @@ def test_workloads_are_seeded_and_shaped():
     n = 512 + w3.text_len
     exp = int((n * n + 64 * n + 2080 + 50 * (n + 114)).sum())
     assert w3.pairs() == exp
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """One GPU is all this build drives: ``bench.py --gpus N`` with N > 1 says so and exits."""
+    import subprocess
+    import sys
+
+    root = Path(__file__).resolve().parent.parent
+    r = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_entry_points_exist():
+    import importlib.util
+
+    root = Path(__file__).resolve().parent.parent
+    spec = importlib.util.spec_from_file_location("graft_entry", root / "__graft_entry__.py")
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    assert callable(mod.build) and callable(mod.smoke)
