@@ -258,7 +258,7 @@ int bcattn_fwd_kvcache(const bcattn_fwd_params *p, void *stream) {
   const size_t R = (size_t)a.G * a.Sq;
   const size_t rows = (size_t)a.B * a.Hkv * s.nsplit * ((R + kSplitRows - 1) / kSplitRows) * kSplitRows;
   s.part_ml = reinterpret_cast<float *>(ws);
-  s.part_o = reinterpret_cast<part_t *>(ws + split_ml_bytes(rows));
+  s.part_o = ws + split_ml_bytes(rows);
   rc = p->dtype == BCATTN_F16 ? f16::launch_fwd_kvcache_mfma(a, s, p->D, st)
                               : bf16::launch_fwd_kvcache_mfma(a, s, p->D, st);
   if (rc) return fail(rc, "kvcache forward launch failed (D=%d)", p->D);

@@ -187,15 +187,16 @@ int launch_fwd_f32(const FwdArgs &a, int D, hipStream_t st);
 int launch_bwd_f32(const BwdArgs &a, int D, hipStream_t st);
 
 // Split-key partials of the KV-cached forward.  A work item is (batch, kv head, split,
-// row tile of kSplitRows packed rows); its head_dim accumulators are stored in the order
-// the lanes hold them.
-typedef float part_t;  // fp32: bf16 partials were measured no faster (the call is latency-bound) and cost accuracy
-typedef f32x4 part4_t;
+// row tile of kSplitRows packed rows).  A partial output is stored normalised by its own row
+// sum (so |value| <= max |v|) in the element type of the call, in the order the lanes hold
+// the accumulators: [wave][head_dim block][pair of register quads][lane][8], i.e. every store
+// and load instruction moves 64 consecutive 16-byte vectors.  (fp32 partials were the larger
+// half of the call's memory traffic.)
 constexpr int kSplitRows = 128;
 constexpr int kSplitTarget = 256;  // workgroups to aim for: one per CU, each holds most of a CU's LDS
 inline size_t split_ml_bytes(size_t rows) { return (rows * 2 * sizeof(float) + 255) & ~(size_t)255; }
 struct SplitArgs {
-  part_t *part_o;  // (B, Hkv, nsplit, row tiles, kSplitRows * D)
+  void *part_o;    // (B, Hkv, nsplit, row tiles, kSplitRows * D), 16-bit elements
   float *part_ml;  // (B, Hkv, nsplit, row tiles, kSplitRows, 2): running max (raw scores), sum
   int nsplit;
   int tiles_per_split;  // 64-key tiles per split

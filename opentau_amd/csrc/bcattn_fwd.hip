@@ -17,7 +17,7 @@ namespace bcattn {
 inline namespace BCATTN_ELEM_NS {
 
 // SPLIT: the key tiles are divided over `nsplit` workgroups per row tile; each
-// writes its unnormalised fp32 partial (O, running max, sum) and
+// writes its partial (O normalised by its own sum, 16-bit; reference point, sum) and
 // `fwd_combine_kernel` merges them.  This is what lets a handful of
 // (batch, kv head) problems with few query rows fill the chip.
 // LDS stages: three where they fit in the 160 KB of a CU, else two.
@@ -365,15 +365,16 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
       ml[1] = has ? l : 0.f;
       *reinterpret_cast<f32x2 *>(sp.part_ml + 2 * (item * BM + wave * 32 + n)) = ml;
     }
-    part_t *po = sp.part_o + item * (BM * D) + (int64_t)wave * (32 * D) + 4 * lane;
+    e16_t *po = reinterpret_cast<e16_t *>(sp.part_o) + item * (BM * D) + (int64_t)wave * (32 * D) + 8 * lane;
+    const float pinv = has ? 1.f / l : 0.f;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        part4_t w;
-#pragma unroll
-        for (int x = 0; x < 4; ++x) w[x] = o[db][4 * r4 + x];
-        *reinterpret_cast<part4_t *>(po + (db * 4 + r4) * 256) = w;
+      for (int rp = 0; rp < 2; ++rp) {
+        const int r0 = 8 * rp;  // register quads 2*rp, 2*rp+1
+        *reinterpret_cast<e16x8 *>(po + (db * 2 + rp) * 512) =
+            pack8(o[db][r0] * pinv, o[db][r0 + 1] * pinv, o[db][r0 + 2] * pinv, o[db][r0 + 3] * pinv,
+                  o[db][r0 + 4] * pinv, o[db][r0 + 5] * pinv, o[db][r0 + 6] * pinv, o[db][r0 + 7] * pinv);
       }
     return;
   }
@@ -401,16 +402,18 @@ constexpr size_t fwd_stage_bytes() {
   return StageLayout<D, (SPLIT ? SplitStages<D>::value : FwdStages<D>::value), 256>::kBytes;
 }
 
-// Merge the per-split partials.  A thread owns the same (wave, head_dim block, register
-// quad, lane) slot the split kernel's lanes wrote, so its loads are consecutive across
-// the wave; blockIdx.x = (batch, kv head, row tile), blockIdx.y = (wave, head_dim block).
+// Merge the per-split partials.  A thread owns the same (wave, head_dim block, pair of register
+// quads, lane) slot the split kernel's lanes wrote, so its loads are consecutive across the
+// wave; blockIdx.x = (batch, kv head, row tile), blockIdx.y = (wave, pair of head_dim blocks);
+// the four waves of a block take (head_dim block of the pair) x (quad pair).
 template <int D, int NW>
 __global__ __launch_bounds__(256) void fwd_combine_kernel(const FwdArgs a, const SplitArgs sp) {
   constexpr int DB = D / 32, BM = 32 * NW;
   const int R = a.G * a.Sq;
   const int ntile_r = (R + BM - 1) / BM;
-  const int lane = threadIdx.x & 63, r4 = threadIdx.x >> 6;
-  const int db = blockIdx.y % DB, wave = blockIdx.y / DB;
+  const int lane = threadIdx.x & 63, sub = threadIdx.x >> 6;
+  const int rp = sub & 1;
+  const int db = 2 * (blockIdx.y % (DB / 2)) + (sub >> 1), wave = blockIdx.y / (DB / 2);
   const int tile = blockIdx.x % ntile_r;
   const int64_t bh = blockIdx.x / ntile_r;
   const int hk = (int)(bh % a.Hkv);
@@ -426,7 +429,8 @@ __global__ __launch_bounds__(256) void fwd_combine_kernel(const FwdArgs a, const
   // Loads go out eight splits at a time (indices past the end repeat the last split
   // and get weight zero): a loop of dependent loads would pay the memory latency per split.
   constexpr int CH = 8;
-  const part_t *pp = sp.part_o + item0 * (BM * D) + (int64_t)wave * (32 * D) + (db * 4 + r4) * 256 + 4 * lane;
+  const e16_t *pp = reinterpret_cast<const e16_t *>(sp.part_o) + item0 * (BM * D) + (int64_t)wave * (32 * D) +
+                    (db * 2 + rp) * 512 + 8 * lane;
   const int64_t po_step = (int64_t)ntile_r * (BM * D);
   float mx = -INFINITY;
   for (int s0 = 0; s0 < sp.nsplit; s0 += CH) {
@@ -436,36 +440,40 @@ __global__ __launch_bounds__(256) void fwd_combine_kernel(const FwdArgs a, const
 #pragma unroll
     for (int j = 0; j < CH; ++j) mx = fmaxf(mx, mv[j]);
   }
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   float lsum = 0.f;
   const float mref = mx == -INFINITY ? 0.f : mx;
   for (int s0 = 0; s0 < sp.nsplit; s0 += CH) {
     f32x2 ml[CH];
-    part4_t po[CH];
+    e16x8 po[CH];
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
       const int sj = min(s0 + j, sp.nsplit - 1);
       ml[j] = *reinterpret_cast<const f32x2 *>(mlp + sj * ml_step);
-      po[j] = *reinterpret_cast<const part4_t *>(pp + sj * po_step);
+      po[j] = *reinterpret_cast<const e16x8 *>(pp + sj * po_step);
     }
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
-      // a split without a visible key has max -inf and sum 0: weight 0, not NaN
+      // a split without a visible key has max -inf and sum 0: weight 0, not NaN;
+      // a partial is normalised by its own sum, so its weight carries that sum
       const bool live = s0 + j < sp.nsplit && ml[j][0] != -INFINITY;
-      const float e = live ? fast_exp2((ml[j][0] - mref) * c) : 0.f;
-      lsum += e * ml[j][1];
+      const float w = live ? fast_exp2((ml[j][0] - mref) * c) * ml[j][1] : 0.f;
+      lsum += w;
 #pragma unroll
-      for (int x = 0; x < 4; ++x) acc[x] += live ? e * po[j][x] : 0.f;
+      for (int x = 0; x < 8; ++x) acc[x] += live ? w * (float)po[j][x] : 0.f;
     }
   }
   const bool has = lsum > 0.f;
   const float inv = has ? 1.f / lsum : 0.f;
-  e16x4 w;
-#pragma unroll
-  for (int x = 0; x < 4; ++x) w[x] = (e16_t)(acc[x] * inv);
   e16_t *optr = reinterpret_cast<e16_t *>(a.o) + b * a.o_sb + (int64_t)i * a.o_ss + h * a.o_sh;
-  *reinterpret_cast<e16x4 *>(optr + 32 * db + 8 * r4 + 4 * hh) = w;
-  if (a.lse != nullptr && db == 0 && r4 == 0 && hh == 0)
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {  // register quads 2*rp + q: head_dim 32*db + 8*(2*rp+q) + 4*hh ..+3
+    e16x4 w;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) w[x] = (e16_t)(acc[4 * q + x] * inv);
+    *reinterpret_cast<e16x4 *>(optr + 32 * db + 8 * (2 * rp + q) + 4 * hh) = w;
+  }
+  if (a.lse != nullptr && db == 0 && rp == 0 && hh == 0)
     a.lse[((int64_t)b * a.H + h) * a.Sq + i] = has ? mx * a.scale + __logf(lsum) : 0.f;
 }
 
@@ -524,7 +532,7 @@ size_t kvcache_workspace_bytes(int B, int Sq, int Sk0, int Sk, int H, int Hkv, i
   if (ns <= 1) return 0;
   const size_t R = (size_t)(H / Hkv) * Sq;
   const size_t rows = (size_t)B * Hkv * ns * ((R + kSplitRows - 1) / kSplitRows) * kSplitRows;
-  return split_ml_bytes(rows) + ((rows * D * sizeof(part_t) + 255) & ~(size_t)255);
+  return split_ml_bytes(rows) + ((rows * D * sizeof(e16_t) + 255) & ~(size_t)255);
 }
 
 template <int D>
@@ -534,7 +542,7 @@ static int launch_split(const FwdArgs &a, const SplitArgs &sp, hipStream_t st) {
   const int rc = launch_fwd_t<D, NW, true>(a, sp, st);
   if (rc) return rc;
   const int ntile_r = (R + kSplitRows - 1) / kSplitRows;
-  hipLaunchKernelGGL((fwd_combine_kernel<D, NW>), dim3((unsigned)(a.B * a.Hkv * ntile_r), NW * (D / 32)),
+  hipLaunchKernelGGL((fwd_combine_kernel<D, NW>), dim3((unsigned)(a.B * a.Hkv * ntile_r), NW * (D / 64)),
                      dim3(256), 0, st, a, sp);
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
 }
