@@ -447,7 +447,10 @@ def test_sequence_beyond_the_tile_table_is_refused():
 # KV-cached suffix call
 # --------------------------------------------------------------------------- #
 @pytest.mark.parametrize("b,sq,h,hkv,d,cross", [(2, 50, 8, 1, 256, 968), (2, 50, 8, 4, 256, 1024),
-                                                (1, 51, 16, 2, 128, 700), (2, 33, 8, 1, 256, 20)])
+                                                (1, 51, 16, 2, 128, 700), (2, 33, 8, 1, 256, 20),
+                                                # caches that end inside a tile, at every head_dim
+                                                (1, 70, 16, 2, 128, 712), (2, 50, 8, 2, 64, 248), (1, 130, 8, 1, 256, 40),
+                                                (1, 50, 8, 1, 256, 969)])
 def test_kvcache_equals_concat(b, sq, h, hkv, d, cross):
     ids = make_blocks(b, sq, "prefixlm", cross=cross)
     q = randn((b, sq, h, d), torch.bfloat16, 1)
