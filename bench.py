@@ -32,9 +32,9 @@ PEAK_HBM_GBPS = 8000.0
 # the same counter reads for a plain 1 GiB device copy (FETCH_SIZE reads half the bytes: factor 2.0;
 # WRITE_SIZE: factor 1.0).  Other workloads have no such measurement and report null.
 HBM_TRAFFIC_BYTES = {
-    ("c5", "fwd"): int((286544.8 * 2.0 + 286134.8) * 1024),
-    ("c5", "bwd_dq"): int((437374.5 * 2.0 + 281728.0) * 1024),
-    ("c5", "bwd_dkv"): int((669672.8 * 2.0 + 70432.0) * 1024),
+    ("c5", "fwd"): int((286503.7 * 2.0 + 286134.8) * 1024),
+    ("c5", "bwd_dq"): int((437434.9 * 2.0 + 281728.0) * 1024),
+    ("c5", "bwd_dkv"): int((675657.6 * 2.0 + 70432.0) * 1024),
 }
 
 
