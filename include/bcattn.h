@@ -52,7 +52,7 @@
 extern "C" {
 #endif
 
-#define BCATTN_ABI_VERSION 1
+#define BCATTN_ABI_VERSION 2
 
 enum bcattn_dtype { BCATTN_F32 = 0, BCATTN_BF16 = 1, BCATTN_F16 = 2 };
 
@@ -98,6 +98,17 @@ typedef struct bcattn_fwd_params {
    * whose mask is identical — and the summary pass is skipped.
    */
   int32_t summary_ready;
+  /*
+   * Best-of-N sampling: every run of kv_share consecutive batch entries reads ONE
+   * batch entry of segment 0 (batch entry b reads k, v at batch index
+   * b / kv_share, so k and v hold B / kv_share entries); 0 or 1: no sharing.
+   * Same result as repeating each cached entry kv_share times along the batch
+   * axis, which is what expand_kv_cache materialises
+   * (src/opentau/policies/candidates.py:114-127, called from
+   * src/opentau/policies/pi05/modeling_pi05.py:2011).  Segment 1, the ids and
+   * the valid flags stay per batch entry.  B must be a multiple of kv_share.
+   */
+  int32_t kv_share;
   void *workspace;
   size_t workspace_bytes;
 } bcattn_fwd_params;

@@ -142,6 +142,8 @@ static int check_fwd(const bcattn_fwd_params *p) {
     return rc;
   if (!p->q_blk || !p->k_blk || !p->q_valid || !p->k_valid)
     return fail(BCATTN_ERR_INVALID, "null block-id / valid pointer");
+  if (p->kv_share < 0 || (p->kv_share > 1 && p->B % p->kv_share))
+    return fail(BCATTN_ERR_INVALID, "kv_share=%d does not divide B=%d", p->kv_share, p->B);
   return BCATTN_OK;
 }
 
@@ -170,6 +172,7 @@ static FwdArgs fwd_args(const bcattn_fwd_params *p) {
   a.H = p->H;
   a.Hkv = p->Hkv;
   a.G = p->H / p->Hkv;
+  a.kv_share = p->Sk0 > 0 && p->kv_share > 1 ? p->kv_share : 1;
   a.scale = p->scale;
   return a;
 }

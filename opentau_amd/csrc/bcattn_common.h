@@ -131,6 +131,7 @@ struct FwdArgs {
   const tile_summary_t *ksum;  // (B, nt): key tiles, segment 0 first, never straddling
   const int32_t *kbm;          // (B, nt, 64): block id per tile slot, INT_MAX where invalid / padding
   int B, Sq, Sk0, Sk, H, Hkv, G;
+  int kv_share;  // >= 1: batch entry b reads segment 0 at batch index b / kv_share
   float scale;
 };
 

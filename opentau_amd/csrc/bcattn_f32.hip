@@ -71,8 +71,8 @@ __global__ __launch_bounds__(256) void fwd_f32_kernel(const FwdArgs a, const int
   for (int x = 0; x < F_BR; ++x) qmax_g = max(qmax_g, red_s[x]);
 
   const int Sk = a.Sk;
-  const float *k0b = reinterpret_cast<const float *>(a.k0.ptr) + b * a.k0.sb + hk * a.k0.sh;
-  const float *v0b = reinterpret_cast<const float *>(a.v0.ptr) + b * a.v0.sb + hk * a.v0.sh;
+  const float *k0b = reinterpret_cast<const float *>(a.k0.ptr) + (b / a.kv_share) * a.k0.sb + hk * a.k0.sh;
+  const float *v0b = reinterpret_cast<const float *>(a.v0.ptr) + (b / a.kv_share) * a.v0.sb + hk * a.v0.sh;
   const float *k1b = reinterpret_cast<const float *>(a.k1.ptr) + b * a.k1.sb + hk * a.k1.sh;
   const float *v1b = reinterpret_cast<const float *>(a.v1.ptr) + b * a.v1.sb + hk * a.v1.sh;
   const int nt0s = (a.Sk0 + kSumTile - 1) / kSumTile;  // summary tiles of segment 0

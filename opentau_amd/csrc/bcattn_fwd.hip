@@ -56,11 +56,17 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
   if (bid >= nitems) return;
   const int tile = __builtin_amdgcn_readfirstlane(bid % ntile_r);
   bid /= ntile_r;
+  // Batch entries that share a cached segment are neighbours in the order of the work
+  // items (same split, same kv head): they stream it through one L2.  (Measured 5 % faster
+  // than leaving them a whole batch entry apart, where every XCD fetches the segment.)
+  const int cand = __builtin_amdgcn_readfirstlane(bid % a.kv_share);
+  bid /= a.kv_share;
   const int split = SPLIT ? __builtin_amdgcn_readfirstlane(bid % sp.nsplit) : 0;
   if (SPLIT) bid /= sp.nsplit;
   // (division results live in vector registers; say that they are uniform)
   const int hk = __builtin_amdgcn_readfirstlane(bid % a.Hkv);
-  const int b = __builtin_amdgcn_readfirstlane(bid / a.Hkv);
+  const int b0 = __builtin_amdgcn_readfirstlane(bid / a.Hkv);  // batch index of segment 0
+  const int b = b0 * a.kv_share + cand;
 
   // Key tiles never straddle the two key segments: tiles [0, nt0) cover segment 0,
   // tiles [nt0, nt0+nt1) segment 1, each padded (zero rows, invalid ids) at its end.
@@ -69,8 +75,8 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
   const int t_first = SPLIT ? split * sp.tiles_per_split : 0;
   const tile_summary_t *ksum = a.ksum + (int64_t)b * nt_all;
 
-  const e16_t *k0b = reinterpret_cast<const e16_t *>(a.k0.ptr) + b * a.k0.sb + hk * a.k0.sh;
-  const e16_t *v0b = reinterpret_cast<const e16_t *>(a.v0.ptr) + b * a.v0.sb + hk * a.v0.sh;
+  const e16_t *k0b = reinterpret_cast<const e16_t *>(a.k0.ptr) + b0 * a.k0.sb + hk * a.k0.sh;
+  const e16_t *v0b = reinterpret_cast<const e16_t *>(a.v0.ptr) + b0 * a.v0.sb + hk * a.v0.sh;
   const e16_t *k1b = reinterpret_cast<const e16_t *>(a.k1.ptr) + b * a.k1.sb + hk * a.k1.sh;
   const e16_t *v1b = reinterpret_cast<const e16_t *>(a.v1.ptr) + b * a.v1.sb + hk * a.v1.sh;
   const int n0 = a.Sk0 > 0 ? a.Sk0 : 1, n1 = a.Sk - a.Sk0 > 0 ? a.Sk - a.Sk0 : 1;

@@ -130,6 +130,23 @@ def _check_inputs(q, k, v):
         raise RuntimeError("q, k, v must be (B, S, H, D)")
 
 
+def _kv_share(b: int, k: torch.Tensor, v: torch.Tensor, k_new: torch.Tensor | None) -> int:
+    """Batch entries of ``q`` per batch entry of key segment 0 (1: the usual one to one)."""
+    bk = k.shape[0]
+    if v.shape[0] != bk:
+        raise RuntimeError(f"k and v differ in batch size: {bk} and {v.shape[0]}")
+    if bk == b:
+        return 1
+    if k_new is None or bk == 0 or b % bk or k.shape[1] == 0:
+        raise RuntimeError(
+            f"k/v batch {bk} does not match q batch {b}; only a cached segment followed by per-entry "
+            "k_new/v_new may be shared, by a whole number of q entries each"
+        )
+    if k_new.shape[0] != b:
+        raise RuntimeError(f"k_new batch {k_new.shape[0]} does not match q batch {b}")
+    return b // bk
+
+
 _MFMA_HEAD_DIMS = (64, 128, 256)
 
 
@@ -169,7 +186,10 @@ def forward_raw(
 
     ``k``/``v`` are key segment 0; ``k_new``/``v_new`` (optional) segment 1.
     ``workspace`` (uint8, device) may be passed to reuse the key-tile summary of
-    an earlier call with the same mask (``summary_ready=True``).
+    an earlier call with the same mask (``summary_ready=True``).  When segment 0
+    has fewer batch entries than ``q`` (``B = n * k.shape[0]``), batch entry ``b``
+    reads entry ``b // n`` of it: the un-expanded prefix cache of best-of-N
+    sampling (``src/opentau/policies/candidates.py:114-127``).
     """
     lib = _loader.require_library()
     _check_inputs(q, k, v)
@@ -184,6 +204,7 @@ def forward_raw(
     b, sq, h, d = q.shape
     sk0, hkv = k.shape[1], k.shape[2]
     sk1 = 0 if k_new is None else k_new.shape[1]
+    share = _kv_share(b, k, v, k_new)
     q, k, v = _operand(q, vec), _operand(k, vec), _operand(v, vec)
     if k_new is not None:
         k_new, v_new = _operand(k_new, vec), _operand(v_new, vec)
@@ -205,6 +226,7 @@ def forward_raw(
     p.B, p.Sq, p.Sk0, p.Sk1, p.H, p.Hkv, p.D = b, sq, sk0, sk1, h, hkv, d
     p.dtype, p.scale = code, float(scale)
     p.summary_ready = 1 if summary_ready else 0
+    p.kv_share = share
     size_fn = lib.bcattn_fwd_kvcache_workspace_bytes if kvcache else lib.bcattn_fwd_workspace_bytes
     need = size_fn(ctypes.byref(p))
     if workspace is None or workspace.numel() < need:
@@ -370,10 +392,16 @@ def _kvc_setup(ctx, inputs, output):
 def _kvc_backward(ctx, d_out, _d_lse):
     q, k_cache, v_cache, k_new, v_new, out, lse, q_blk, k_blk, q_valid, k_valid = ctx.saved_tensors
     n0 = k_cache.shape[1]
+    share = q.shape[0] // k_cache.shape[0]
+    if share > 1:  # a shared cache entry collects the gradients of all the entries that read it
+        k_cache, v_cache = (t.repeat_interleave(share, dim=0) for t in (k_cache, v_cache))
     k = torch.cat([k_cache, k_new], dim=1)
     v = torch.cat([v_cache, v_new], dim=1)
     dq, dk, dv = _op_bwd(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, ctx.scale)
-    return dq, dk[:, :n0], dv[:, :n0], dk[:, n0:], dv[:, n0:], None, None, None, None, None
+    dkc, dvc = dk[:, :n0], dv[:, :n0]
+    if share > 1:
+        dkc, dvc = (t.reshape(-1, share, *t.shape[1:]).float().sum(1).to(t.dtype) for t in (dkc, dvc))
+    return dq, dkc, dvc, dk[:, n0:], dv[:, n0:], None, None, None, None, None
 
 
 _op_fwd_kvcache.register_autograd(_kvc_backward, setup_context=_kvc_setup)
@@ -424,6 +452,11 @@ def flash_attn_blockmask_kvcache(
     ``k_blk``/``k_valid`` covering the concatenation (cached columns carry
     ``INT_BLK_MIN``), which is what the reference computes per layer and denoise
     step (``src/opentau/policies/pi05/paligemma_with_expert.py:742-768``).
+
+    ``k_cache``/``v_cache`` may hold ``B / n`` batch entries: entry ``b`` of ``q`` then
+    attends cache entry ``b // n``, the ``(b n)`` order of best-of-N sampling, without
+    the ``n`` copies of the prefix cache that ``expand_kv_cache`` makes
+    (``src/opentau/policies/candidates.py:114-127``).
     """
     if _needs_graph(q, k_cache, v_cache, k_new, v_new):
         return _op_fwd_kvcache(q, k_cache, v_cache, k_new, v_new, q_blk, k_blk, q_valid, k_valid, float(scale))[0]

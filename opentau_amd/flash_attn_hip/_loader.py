@@ -17,7 +17,7 @@ from pathlib import Path
 
 CSRC = Path(__file__).resolve().parent.parent / "csrc"
 LIB_PATH = CSRC / "libbcattn.so"
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 # status codes of include/bcattn.h
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_LAUNCH = 0, -1, -2, -3, -4
@@ -72,6 +72,7 @@ class FwdParams(ctypes.Structure):
         ("dtype", ctypes.c_int32),
         ("scale", ctypes.c_float),
         ("summary_ready", ctypes.c_int32),
+        ("kv_share", ctypes.c_int32),
         ("workspace", ctypes.c_void_p),
         ("workspace_bytes", ctypes.c_size_t),
     ]

@@ -3,6 +3,7 @@ symbol the header declares, and the Python surface fails loudly without a GPU.""
 
 import ctypes
 import re
+import subprocess
 from pathlib import Path
 
 import pytest
@@ -31,11 +32,29 @@ def test_library_loads_and_exports_every_declared_symbol():
     assert lib.bcattn_abi_version() == _loader.ABI_VERSION
 
 
-def test_struct_layout_matches_header_sizes():
-    # bcattn_tensor: pointer + 3 x int64; params: see include/bcattn.h
+def test_struct_layout_matches_header(tmp_path):
+    """Sizes and field offsets of the ctypes mirrors against what a C compiler makes of include/bcattn.h."""
+    fields = {
+        "bcattn_tensor": (_loader.Tensor4, ["ptr", "stride_b", "stride_s", "stride_h"]),
+        "bcattn_fwd_params": (_loader.FwdParams, [f[0] for f in _loader.FwdParams._fields_]),
+        "bcattn_bwd_params": (_loader.BwdParams, [f[0] for f in _loader.BwdParams._fields_]),
+    }
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "bcattn.h"', "int main(void) {"]
+    for cname, (_, names) in fields.items():
+        lines.append(f'  printf("{cname} %zu\\n", sizeof({cname}));')
+        lines += [f'  printf("{cname}.{n} %zu\\n", offsetof({cname}, {n}));' for n in names]
+    lines += ["  return 0;", "}"]
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-I", str(ROOT / "include"), "-o", str(exe), str(src)], check=True)
+    want = dict(line.split() for line in subprocess.run([str(exe)], check=True, capture_output=True,
+                                                        text=True).stdout.splitlines())
     assert ctypes.sizeof(_loader.Tensor4) == 32
-    assert ctypes.sizeof(_loader.FwdParams) == 6 * 32 + 5 * 8 + 7 * 4 + 4 + 4 + 4 + 8 + 8
-    assert ctypes.sizeof(_loader.BwdParams) == 8 * 32 + 5 * 8 + 6 * 4 + 4 + 4 + 4 + 4 + 8 + 8
+    for cname, (ctype, names) in fields.items():
+        assert ctypes.sizeof(ctype) == int(want[cname]), cname
+        for n in names:
+            assert getattr(ctype, n).offset == int(want[f"{cname}.{n}"]), f"{cname}.{n}"
 
 
 def test_workspace_queries_run_without_a_gpu():

@@ -474,6 +474,68 @@ def test_kvcache_equals_concat(b, sq, h, hkv, d, cross):
     assert o_model.shape == (b, sq, h * d) and torch.equal(o_model.reshape(o_split.shape), o_split)
 
 
+@pytest.mark.parametrize("bsrc,n,sq,h,hkv,d,cross,dtype", [
+    (1, 8, 50, 8, 1, 256, 712, torch.bfloat16),   # pi0.5 serving: one observation, 8 candidates
+    (2, 4, 50, 8, 1, 256, 300, torch.bfloat16),   # (b n) order with more than one observation
+    (3, 2, 33, 16, 2, 128, 200, torch.float16),
+    (2, 3, 20, 4, 2, 64, 70, torch.float32),
+])
+def test_kvcache_shared_across_candidates(bsrc, n, sq, h, hkv, d, cross, dtype):
+    """Best-of-N sampling: every run of n batch entries reads one entry of the prefix cache.  The
+    result is that of the cache repeated n times along the batch axis (what the reference's
+    expand_kv_cache materialises, candidates.py:114-127), bit for bit, in all three forward calls."""
+    b = bsrc * n
+    ids = make_blocks(b, sq, "prefixlm", cross=cross)
+    q = randn((b, sq, h, d), dtype, 1)
+    kc, vc = randn((bsrc, cross, hkv, d), dtype, 2), randn((bsrc, cross, hkv, d), dtype, 3)
+    kn, vn = randn((b, sq, hkv, d), dtype, 4), randn((b, sq, hkv, d), dtype, 5)
+    kx, vx = kc.repeat_interleave(n, dim=0), vc.repeat_interleave(n, dim=0)
+    ref = eager.eager_from_block_ids(q, torch.cat([kx, kn], 1), torch.cat([vx, vn], 1), *ids, d**-0.5).float()
+    gi = [g(t) for t in ids]
+    for kvcache in (True, False):
+        o_sh, l_sh = fa.forward_raw(g(q), g(kc), g(vc), *gi, d**-0.5, g(kn), g(vn), kvcache=kvcache)
+        o_ex, l_ex = fa.forward_raw(g(q), g(kx), g(vx), *gi, d**-0.5, g(kn), g(vn), kvcache=kvcache)
+        assert torch.equal(o_sh, o_ex) and torch.equal(l_sh, l_ex)
+        if dtype == torch.float32:
+            assert rel_l2(o_sh.cpu(), ref) <= 1e-5
+        else:
+            assert_close_bf16(o_sh.float().cpu(), ref, "shared cache out")
+    o_model = attention.flash_attention_forward_kvcache(None, gi, b, d, g(q), g(kc), g(vc), g(kn), g(vn))
+    assert torch.equal(o_model.reshape(o_sh.shape), fa.forward_raw(g(q), g(kc), g(vc), *gi, d**-0.5, g(kn), g(vn),
+                                                                   kvcache=True)[0])
+
+
+def test_kvcache_shared_gradients_sum_over_candidates():
+    bsrc, n, sq, h, hkv, d, cross = 2, 3, 40, 8, 2, 128, 150
+    b = bsrc * n
+    gi = [g(t) for t in make_blocks(b, sq, "prefixlm", cross=cross)]
+    mk = lambda shape, seed: g(randn(shape, torch.bfloat16, seed)).requires_grad_(True)  # noqa: E731
+    q, kc, vc = mk((b, sq, h, d), 1), mk((bsrc, cross, hkv, d), 2), mk((bsrc, cross, hkv, d), 3)
+    kn, vn = mk((b, sq, hkv, d), 4), mk((b, sq, hkv, d), 5)
+    w = g(randn((b, sq, h, d), torch.bfloat16, 6))
+    (fa.flash_attn_blockmask_kvcache(q, kc, vc, kn, vn, *gi, d**-0.5).float() * w.float()).sum().backward()
+    got = [t.grad.clone() for t in (q, kc, vc, kn, vn)]
+    for t in (q, kc, vc, kn, vn):
+        t.grad = None
+    kx, vx = kc.repeat_interleave(n, dim=0), vc.repeat_interleave(n, dim=0)  # autograd sums over the copies
+    (fa.flash_attn_blockmask_kvcache(q, kx, vx, kn, vn, *gi, d**-0.5).float() * w.float()).sum().backward()
+    want = [t.grad for t in (q, kc, vc, kn, vn)]
+    for name, a, e in zip(("dq", "dk_cache", "dv_cache", "dk_new", "dv_new"), got, want):
+        assert_close_bf16(a.float().cpu(), e.float().cpu(), name)
+
+
+def test_kvcache_share_must_divide_batch():
+    d = 64
+    gi = [g(t) for t in make_blocks(3, 8, "prefixlm", cross=16)]
+    q = g(randn((3, 8, 2, d), torch.bfloat16, 1))
+    kc = g(randn((2, 16, 2, d), torch.bfloat16, 2))
+    kn = g(randn((3, 8, 2, d), torch.bfloat16, 3))
+    with pytest.raises(RuntimeError, match="batch"):
+        fa.forward_raw(q, kc, kc, *gi, d**-0.5, kn, kn, kvcache=True)
+    with pytest.raises(RuntimeError, match="batch"):  # sharing needs the per-entry second segment
+        fa.forward_raw(q, kc[:1], kc[:1], gi[0], gi[1][:, :16], gi[2], gi[3][:, :16], d**-0.5)
+
+
 def test_kvcache_summary_reuse_across_layers():
     b, sq, h, hkv, d, cross = 2, 50, 8, 1, 256, 300
     ids = [g(t) for t in make_blocks(b, sq, "prefixlm", cross=cross)]
