@@ -52,6 +52,8 @@ def main() -> int:
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="only run a plain device copy of MIB MiB a few times (reference for the "
                          "FETCH_SIZE / WRITE_SIZE counters) and exit")
+    ap.add_argument("--rope-only", action="store_true",
+                    help="only run the rotary-embedding leg and print its record (for profiles of that kernel)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1",
@@ -72,6 +74,9 @@ def main() -> int:
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.rope_only:
+        print(json.dumps({"rope": bench_rope(torch, dev)}))
+        return 0
     if args.copy_calibration:
         n = args.copy_calibration << 20
         src = torch.empty(n, dtype=torch.uint8, device=dev).fill_(1)
@@ -177,6 +182,7 @@ def main() -> int:
         result["denoise"] = bench_denoise(torch, fa, make_denoise_workload, dev)
         if args.workload == "c5" and not args.no_others:
             result["other_workloads"] = {n: bench_step_only(torch, fa, make_workload, dev, n) for n in ("c3", "c4")}
+            result["rope"] = bench_rope(torch, dev)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, make_workload, args.workload)
     print(json.dumps(result))
@@ -213,6 +219,40 @@ def bench_step_only(torch, fa, make_workload, dev, name, steps=20, warmup=3):
         "tflops": round(flops / (ms * 1e-3) / 1e12, 2),
         "pct_of_bf16_mfma_peak": round(100 * flops / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 2),
     }
+
+
+def bench_rope(torch, dev, calls=50, warmup=5):
+    """The rotary-embedding pass that feeds the attention call (queries and keys of one layer,
+    in place, bf16), at the training shapes: an HBM-bound kernel, so GB/s on its algorithmic
+    bytes (every element read once and written once, plus the positions) against the HBM peak."""
+    from opentau_amd import rope
+
+    out = {}
+    for name, (b, length, h, hkv, d) in {"c3": (32, 754, 8, 1, 256), "c5": (4, 4402, 64, 8, 128)}.items():
+        gen = torch.Generator(device="cpu").manual_seed(0)
+        q = torch.randn(b, length, h, d, generator=gen).to(dev, torch.bfloat16)
+        k = torch.randn(b, length, hkv, d, generator=gen).to(dev, torch.bfloat16)
+        pos = torch.arange(length, dtype=torch.int32, device=dev)[None].expand(b, length).contiguous()
+        for _ in range(warmup):
+            rope.rope_raw(q, k, pos, q_out=q, k_out=k)
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0.record()
+        for _ in range(calls):
+            rope.rope_raw(q, k, pos, q_out=q, k_out=k)
+        t1.record()
+        torch.cuda.synchronize()
+        us = t0.elapsed_time(t1) * 1e3 / calls
+        nbytes = 2 * 2 * (q.numel() + k.numel()) + 4 * pos.numel()
+        gbps = nbytes / (us * 1e-6) / 1e9
+        out[name] = {
+            "workload": f"rope of q and k in place, bf16 B{b} L{length} H{h} Hkv{hkv} D{d}",
+            "us_per_call": round(us, 2),
+            "algorithmic_bytes": nbytes,
+            "gbps": round(gbps, 1),
+            "hbm_frac": round(gbps / PEAK_HBM_GBPS, 4),
+        }
+    return out
 
 
 def bench_denoise(torch, fa, make_denoise_workload, dev):

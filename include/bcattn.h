@@ -175,6 +175,44 @@ int bcattn_fwd_kvcache(const bcattn_fwd_params *p, void *stream);
 /* Replaces flash_bwd (flash_blockmask.cu:1210-1327). */
 int bcattn_bwd(const bcattn_bwd_params *p, void *stream);
 
+/*
+ * Rotary position embedding of a layer's queries and keys in one launch, with an
+ * optional per-head RMS norm in front of it.  Replaces the two apply_rope calls
+ * of src/opentau/policies/pi05/paligemma_with_expert.py:739-740 (the function:
+ * :52-107) and, with norm weights, Gemma-3's q_norm / k_norm followed by
+ * apply_rope (src/opentau/policies/pi06/gemma3_with_expert.py:851-861).
+ *
+ * Element d < D/2 of a row pairs with element d + D/2; band d turns by
+ *     angle = position / timescale[d],   timescale[d] = max_wavelength ** (2 d / D)
+ *     out[d]       = x[d] * cos(angle) - x[d + D/2] * sin(angle)
+ *     out[d + D/2] = x[d + D/2] * cos(angle) + x[d] * sin(angle)
+ * in fp32, rounded once to the element type, as the reference does.  The caller
+ * supplies the D/2 timescales (so they are the very numbers its framework
+ * computes).  With n_axes > 1 (interleaved MRoPE) band d reads the position of
+ * axis d % n_axes.  The norm, when asked for, is Gemma-3's: x * rsqrt(mean(x^2) +
+ * eps) * (1 + w), rounded to the element type before the rotation.
+ *
+ * An output may be its input (in place), or any other strided tensor: e.g. the
+ * rows of a preallocated key cache that this layer's keys belong in.
+ * Supported: D % 16 == 0 (D % 8 == 0 for fp32), D <= 512; with a norm D must be
+ * a power of two.  No workspace.
+ */
+typedef struct bcattn_rope_params {
+  bcattn_tensor q, k;         /* (B,L,H,D), (B,L,Hkv,D) in; either pointer may be null: that tensor is skipped */
+  bcattn_tensor q_out, k_out; /* same shapes, out */
+  const int32_t *positions;   /* (n_axes, B, L) contiguous */
+  const float *timescale;     /* (D/2) */
+  const void *q_norm_weight;  /* (D) in the element type of the call, or null: no norm on q */
+  const void *k_norm_weight;  /* likewise for k */
+  int32_t B, L, H, Hkv, D;
+  int32_t n_axes;
+  int32_t dtype;              /* enum bcattn_dtype */
+  int32_t inverse;            /* nonzero: turn by minus the angle, which maps an output gradient to the input gradient; no norm then */
+  float norm_eps;
+} bcattn_rope_params;
+
+int bcattn_rope(const bcattn_rope_params *p, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -337,4 +337,53 @@ int bcattn_bwd(const bcattn_bwd_params *p, void *stream) {
   return BCATTN_OK;
 }
 
+int bcattn_rope(const bcattn_rope_params *p, void *stream) {
+  if (p == nullptr) return fail(BCATTN_ERR_INVALID, "null params");
+  if (p->dtype != BCATTN_F32 && !is16(p->dtype))
+    return fail(BCATTN_ERR_UNSUPPORTED, "dtype %d not supported (0 = fp32, 1 = bf16, 2 = fp16)", p->dtype);
+  const int vec = is16(p->dtype) ? 8 : 4;
+  if (p->B < 0 || p->L < 0 || p->D <= 0 || p->n_axes < 1)
+    return fail(BCATTN_ERR_INVALID, "bad shape B=%d L=%d D=%d n_axes=%d", p->B, p->L, p->D, p->n_axes);
+  if ((int64_t)p->B * p->L >= ((int64_t)1 << 31) - 64) return fail(BCATTN_ERR_UNSUPPORTED, "B*L too large");
+  if (p->D % (2 * vec) || p->D > 512)
+    return fail(BCATTN_ERR_UNSUPPORTED, "rope needs head_dim %% %d == 0 and <= 512; got %d", 2 * vec, p->D);
+  if (p->positions == nullptr || p->timescale == nullptr)
+    return fail(BCATTN_ERR_INVALID, "null positions / timescale pointer");
+  if (!aligned16(p->timescale)) return fail(BCATTN_ERR_INVALID, "timescale: pointer not 16-byte aligned");
+  const bool norm = p->q_norm_weight != nullptr || p->k_norm_weight != nullptr;
+  if (norm && (p->D & (p->D - 1)))
+    return fail(BCATTN_ERR_UNSUPPORTED, "the fused norm needs a power-of-two head_dim; got %d", p->D);
+  if (norm && p->inverse) return fail(BCATTN_ERR_INVALID, "inverse rotation takes no norm");
+  if (norm && !(p->norm_eps >= 0.f)) return fail(BCATTN_ERR_INVALID, "norm_eps must be non-negative");
+  if ((p->q_norm_weight && !aligned16(p->q_norm_weight)) || (p->k_norm_weight && !aligned16(p->k_norm_weight)))
+    return fail(BCATTN_ERR_INVALID, "norm weight: pointer not 16-byte aligned");
+  int rc;
+  if ((rc = check_tensor("q", p->q, vec, false)) || (rc = check_tensor("k", p->k, vec, false))) return rc;
+  if ((rc = check_tensor("q_out", p->q_out, vec, p->q.ptr != nullptr)) ||
+      (rc = check_tensor("k_out", p->k_out, vec, p->k.ptr != nullptr)))
+    return rc;
+  if ((p->q.ptr && p->H <= 0) || (p->k.ptr && p->Hkv <= 0))
+    return fail(BCATTN_ERR_INVALID, "bad head counts H=%d Hkv=%d", p->H, p->Hkv);
+  RopeArgs a;
+  a.q = targ(p->q);
+  a.k = targ(p->k);
+  a.q_out = targ(p->q_out);
+  a.k_out = targ(p->k_out);
+  a.positions = p->positions;
+  a.timescale = p->timescale;
+  a.q_w = p->q.ptr ? p->q_norm_weight : nullptr;
+  a.k_w = p->k.ptr ? p->k_norm_weight : nullptr;
+  a.B = p->B;
+  a.L = p->L;
+  a.H = p->H;
+  a.Hkv = p->Hkv;
+  a.D = p->D;
+  a.n_axes = p->n_axes;
+  a.inverse = p->inverse != 0;
+  a.eps = p->norm_eps;
+  if (launch_rope(a, p->dtype, static_cast<hipStream_t>(stream)))
+    return fail(BCATTN_ERR_LAUNCH, "rope launch failed: %s", hipGetErrorString(hipGetLastError()));
+  return BCATTN_OK;
+}
+
 }  // extern "C"

@@ -154,6 +154,16 @@ struct BwdArgs {
   int stages;  // bit set of bcattn_bwd_stage, never 0 here
 };
 
+struct RopeArgs {
+  TensorArg q, k, q_out, k_out;  // a null ptr skips the tensor
+  const int32_t *positions;      // (n_axes, B, L)
+  const float *timescale;        // (D/2)
+  const void *q_w, *k_w;         // norm weights (D) or null
+  int B, L, H, Hkv, D, n_axes, inverse;
+  float eps;
+};
+int launch_rope(const RopeArgs &a, int dtype, hipStream_t st);
+
 // Lets a kernel use more than 64 KB of dynamic LDS.  The attribute is per device, so a
 // bit per device remembers where it is already set and launches skip the runtime call.
 template <auto Kernel>

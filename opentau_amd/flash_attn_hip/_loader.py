@@ -33,6 +33,7 @@ EXPORTS = (
     "bcattn_fwd",
     "bcattn_fwd_kvcache",
     "bcattn_bwd",
+    "bcattn_rope",
 )
 
 
@@ -110,6 +111,30 @@ class BwdParams(ctypes.Structure):
     ]
 
 
+class RopeParams(ctypes.Structure):
+    """``bcattn_rope_params``."""
+
+    _fields_ = [
+        ("q", Tensor4),
+        ("k", Tensor4),
+        ("q_out", Tensor4),
+        ("k_out", Tensor4),
+        ("positions", ctypes.c_void_p),
+        ("timescale", ctypes.c_void_p),
+        ("q_norm_weight", ctypes.c_void_p),
+        ("k_norm_weight", ctypes.c_void_p),
+        ("B", ctypes.c_int32),
+        ("L", ctypes.c_int32),
+        ("H", ctypes.c_int32),
+        ("Hkv", ctypes.c_int32),
+        ("D", ctypes.c_int32),
+        ("n_axes", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("inverse", ctypes.c_int32),
+        ("norm_eps", ctypes.c_float),
+    ]
+
+
 _lock = threading.Lock()
 _lib = None
 _load_attempted = False
@@ -129,7 +154,8 @@ def _bind(lib: ctypes.CDLL) -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = ctypes.c_size_t
         fn.argtypes = [ctypes.POINTER(st)]
-    for name, st in (("bcattn_fwd", FwdParams), ("bcattn_fwd_kvcache", FwdParams), ("bcattn_bwd", BwdParams)):
+    for name, st in (("bcattn_fwd", FwdParams), ("bcattn_fwd_kvcache", FwdParams), ("bcattn_bwd", BwdParams),
+                     ("bcattn_rope", RopeParams)):
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(st), ctypes.c_void_p]

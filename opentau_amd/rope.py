@@ -1,0 +1,178 @@
+"""Rotary position embedding of a layer's queries and keys on the HIP kernel.
+
+``apply_rope`` has the signature and the numerics of the reference's function of
+that name (``src/opentau/policies/pi05/paligemma_with_expert.py:52-107``; the same
+function serves pi0, pi06 and pi07).  ``apply_rope_qk`` is the form a layer wants:
+queries and keys in one launch, optionally behind Gemma-3's per-head RMS norm
+(``src/opentau/policies/pi06/gemma3_with_expert.py:851-861``), optionally written
+straight into other storage such as the rows of a preallocated key cache.
+There is no CPU path: without the library or a HIP device the calls raise.
+"""
+
+from __future__ import annotations
+
+import ctypes
+
+import torch
+
+from .flash_attn_hip import _loader
+from .flash_attn_hip import _check, _DTYPES, _stream, _t4
+
+_timescales: dict[tuple, torch.Tensor] = {}
+
+
+def rope_timescale(head_dim: int, max_wavelength: float, device: torch.device) -> torch.Tensor:
+    """``max_wavelength ** (2 i / head_dim)`` for the ``head_dim / 2`` bands, fp32, computed with the
+    same torch ops on the same device as ``paligemma_with_expert.py:84-85`` so the kernel divides
+    by the very numbers the reference does.  Cached per (head_dim, wavelength, device)."""
+    key = (head_dim, max_wavelength, str(device))
+    t = _timescales.get(key)
+    if t is None:
+        exponents = (2.0 / head_dim) * torch.arange(head_dim // 2, dtype=torch.float32, device=device)
+        t = (max_wavelength**exponents).to(torch.float32).contiguous()
+        _timescales[key] = t
+    return t
+
+
+def _strided(t: torch.Tensor | None, vec: int, what: str) -> torch.Tensor | None:
+    if t is None:
+        return None
+    if t.ndim != 4:
+        raise RuntimeError(f"{what} must be (B, L, H, D), got {tuple(t.shape)}")
+    if t.stride(-1) != 1 or t.data_ptr() % 16 or any(s % vec for s in t.stride()[:-1]):
+        raise RuntimeError(f"{what}: the head_dim axis must be contiguous, the pointer 16-byte aligned and the "
+                           f"other strides multiples of {vec} elements")
+    return t
+
+
+def _positions(positions: torch.Tensor, b: int, length: int) -> tuple[torch.Tensor, int]:
+    if positions.ndim == 2:
+        n_axes = 1
+    elif positions.ndim == 3:
+        n_axes = positions.shape[0]
+    else:
+        raise RuntimeError(f"positions must be (B, L) or (A, B, L), got {tuple(positions.shape)}")
+    if tuple(positions.shape[-2:]) != (b, length):
+        raise RuntimeError(f"positions {tuple(positions.shape)} do not match (B, L) = {(b, length)}")
+    if positions.is_floating_point():
+        raise RuntimeError("positions must be integers")
+    return positions.to(torch.int32).contiguous(), n_axes
+
+
+def rope_raw(
+    q: torch.Tensor | None,
+    k: torch.Tensor | None,
+    positions: torch.Tensor,
+    max_wavelength: float = 10_000,
+    *,
+    q_out: torch.Tensor | None = None,
+    k_out: torch.Tensor | None = None,
+    q_norm_weight: torch.Tensor | None = None,
+    k_norm_weight: torch.Tensor | None = None,
+    norm_eps: float = 1e-6,
+    inverse: bool = False,
+):
+    """One call of ``bcattn_rope``.  Returns ``(q_out, k_out)`` (``None`` where the input is ``None``)."""
+    lib = _loader.require_library()
+    x = q if q is not None else k
+    if x is None:
+        raise RuntimeError("rope needs q or k")
+    if not x.is_cuda:
+        raise RuntimeError("rope needs tensors on a HIP device; there is no CPU fallback")
+    if x.dtype not in _DTYPES:
+        raise RuntimeError(f"rope supports float32, bfloat16 and float16, got {x.dtype}")
+    code, vec = _DTYPES[x.dtype]
+    q, k = _strided(q, vec, "q"), _strided(k, vec, "k")
+    b, length, d = x.shape[0], x.shape[1], x.shape[3]
+    if q is not None and k is not None and (k.shape[0], k.shape[1], k.shape[3], k.dtype) != (b, length, d, q.dtype):
+        raise RuntimeError(f"q {tuple(q.shape)} and k {tuple(k.shape)} differ in batch, length, head_dim or dtype")
+    pos, n_axes = _positions(positions, b, length)
+    if q is not None and q_out is None:
+        q_out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    if k is not None and k_out is None:
+        k_out = torch.empty(k.shape, dtype=k.dtype, device=k.device)
+    for t, o, what in ((q, q_out, "q_out"), (k, k_out, "k_out")):
+        if t is not None and (_strided(o, vec, what).shape != t.shape or o.dtype != t.dtype or o.device != t.device):
+            raise RuntimeError(f"{what} must have the shape, dtype and device of its input")
+    weights = []
+    for t, w, what in ((q, q_norm_weight, "q_norm_weight"), (k, k_norm_weight, "k_norm_weight")):
+        if w is not None and t is not None:
+            if w.shape != (d,):
+                raise RuntimeError(f"{what} must be ({d},), got {tuple(w.shape)}")
+            w = w.detach().to(device=t.device, dtype=t.dtype).contiguous()
+        weights.append(w if t is not None else None)
+    ts = rope_timescale(d, max_wavelength, x.device)
+    p = _loader.RopeParams()
+    p.q, p.k, p.q_out, p.k_out = _t4(q), _t4(k), _t4(q_out if q is not None else None), _t4(k_out if k is not None else None)
+    p.positions, p.timescale = pos.data_ptr(), ts.data_ptr()
+    p.q_norm_weight = weights[0].data_ptr() if weights[0] is not None else None
+    p.k_norm_weight = weights[1].data_ptr() if weights[1] is not None else None
+    p.B, p.L, p.D = b, length, d
+    p.H = q.shape[2] if q is not None else 0
+    p.Hkv = k.shape[2] if k is not None else 0
+    p.n_axes, p.dtype, p.inverse, p.norm_eps = n_axes, code, 1 if inverse else 0, float(norm_eps)
+    with torch.cuda.device(x.device):
+        _check(lib.bcattn_rope(ctypes.byref(p), _stream(x.device)), lib)
+    return (q_out if q is not None else None), (k_out if k is not None else None)
+
+
+class _Rope(torch.autograd.Function):
+    """The rotation is orthogonal: its gradient is the rotation by minus the angle."""
+
+    @staticmethod
+    def forward(ctx, q, k, positions, max_wavelength):
+        ctx.save_for_backward(positions)
+        ctx.max_wavelength = max_wavelength
+        ctx.has = (q is not None, k is not None)
+        qo, ko = rope_raw(q, k, positions, max_wavelength)
+        return tuple(t for t in (qo, ko) if t is not None)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        (positions,) = ctx.saved_tensors
+        it = iter(grads)
+        gq = next(it).contiguous() if ctx.has[0] else None
+        gk = next(it).contiguous() if ctx.has[1] else None
+        dq, dk = rope_raw(gq, gk, positions, ctx.max_wavelength, inverse=True)
+        return dq, dk, None, None
+
+
+def apply_rope(x: torch.Tensor, positions: torch.Tensor, max_wavelength: float = 10_000) -> torch.Tensor:
+    """``x (B, L, H, D)``, ``positions (B, L)`` or ``(A, B, L)`` -> rotated ``x``, same dtype.
+
+    Drop-in for ``apply_rope`` of ``src/opentau/policies/pi05/paligemma_with_expert.py:52-107``:
+    fp32 arithmetic, one rounding to ``x.dtype``; with 3-D positions band ``i`` follows axis
+    ``i % A`` (interleaved MRoPE).  Differentiable in ``x``.
+    """
+    if torch.is_grad_enabled() and x.requires_grad:
+        return _Rope.apply(x, None, positions, max_wavelength)[0]
+    return rope_raw(x, None, positions, max_wavelength)[0]
+
+
+def apply_rope_qk(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    positions: torch.Tensor,
+    max_wavelength: float = 10_000,
+    *,
+    q_norm_weight: torch.Tensor | None = None,
+    k_norm_weight: torch.Tensor | None = None,
+    norm_eps: float = 1e-6,
+    q_out: torch.Tensor | None = None,
+    k_out: torch.Tensor | None = None,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """Both ``apply_rope`` calls of a layer (``paligemma_with_expert.py:739-740``) in one launch.
+
+    With norm weights: ``apply_rope(q_norm(q), ...)`` and ``apply_rope(k_norm(k), ...)`` of
+    ``src/opentau/policies/pi06/gemma3_with_expert.py:851-861`` where the norms are Gemma-3's
+    (``x * rsqrt(mean(x^2) + eps) * (1 + weight)``, rounded to ``x.dtype``); that form is
+    inference-only.  ``q_out`` / ``k_out`` may be the inputs themselves (in place) or views of
+    other storage, e.g. ``cache_k[:, n0:n0 + L]`` of a preallocated key cache.
+    """
+    norm = q_norm_weight is not None or k_norm_weight is not None
+    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad):
+        if norm or q_out is not None or k_out is not None:
+            raise RuntimeError("apply_rope_qk is differentiable only without norm weights and output arguments")
+        return _Rope.apply(q, k, positions, max_wavelength)
+    return rope_raw(q, k, positions, max_wavelength, q_out=q_out, k_out=k_out, q_norm_weight=q_norm_weight,
+                    k_norm_weight=k_norm_weight, norm_eps=norm_eps)

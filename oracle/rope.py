@@ -1,0 +1,83 @@
+"""CPU oracle for the rotary position embedding (and the per-head RMS norm that can precede it).
+TEST INFRASTRUCTURE ONLY: nothing in the product package may import this module; ``tests/`` and
+the ``cpu_baseline`` leg of ``bench.py`` use it as the checker.
+
+``apply_rope`` restates ``apply_rope`` of the reference
+(``src/opentau/policies/pi05/paligemma_with_expert.py:52-107``; pi0, pi06 and pi07 carry the same
+function) in plain PyTorch, so it runs on CPU or on a GPU tensor alike.  ``gemma3_rms_norm``
+restates ``Gemma3RMSNorm.forward`` of the third-party dependency ``transformers`` (pinned
+``>=4.57,<4.58`` by the reference's ``pyproject.toml:79``; the reference calls it as
+``layer.self_attn.q_norm`` / ``k_norm`` at ``src/opentau/policies/pi06/gemma3_with_expert.py:851-861``).
+
+What pins them (``tests/test_oracle_rope.py``):
+
+* ``apply_rope``       the reference's own tests (``tests/policies/test_pi06.py:159-180``: shape and
+                       dtype kept, different wavelengths differ, position 0 is the identity); the
+                       closed form ``(x1 + i x2) * exp(i * pos / w**(2d/D))`` evaluated in float64 with
+                       Python complex numbers, per element (``rope_closed_form``), which fixes the
+                       pairing d <-> d + D/2, the sign of the rotation and the frequency of every band;
+                       |x1|^2 + |x2|^2 kept; rotations compose by adding positions; the docstring's
+                       claim that equal MRoPE axes reproduce 1-D RoPE bit for bit (``:62-64``); distinct
+                       axes against the closed form (band d follows axis d % A).
+* ``gemma3_rms_norm``  float64 closed form; weight 0 on unit-RMS rows is the identity; a scaled row
+                       gives the same result (scale invariance up to eps).
+
+No function here is "parity unpinned".
+"""
+
+from __future__ import annotations
+
+import cmath
+
+import torch
+
+
+def apply_rope(x: torch.Tensor, positions: torch.Tensor, max_wavelength: float = 10_000) -> torch.Tensor:
+    """``x (B, L, H, D)``; ``positions (B, L)`` or ``(A, B, L)``.  fp32 arithmetic, result in ``x.dtype``
+    (reference ``paligemma_with_expert.py:79-107``)."""
+    d = x.shape[-1]
+    half = d // 2
+    xf = x.to(torch.float32)
+    band = torch.arange(half, dtype=torch.float32, device=x.device)
+    timescale = max_wavelength ** ((2.0 / d) * band)  # :84-85
+    pos = positions.to(torch.float32)
+    if positions.ndim == 3:  # interleaved MRoPE: band i follows axis i % A (:90-97)
+        axis_of_band = torch.arange(half, device=x.device) % positions.shape[0]
+        pos = pos[axis_of_band].permute(1, 2, 0)  # (B, L, half)
+    else:
+        pos = pos.unsqueeze(-1)
+    angle = (pos / timescale).unsqueeze(-2)  # one angle per (token, band), shared by the heads (:99)
+    s, c = torch.sin(angle), torch.cos(angle)
+    lo, hi = xf[..., :half], xf[..., half:]
+    out = torch.cat([lo * c - hi * s, hi * c + lo * s], dim=-1)  # :104-105
+    return out.to(x.dtype)
+
+
+def gemma3_rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    """``x * rsqrt(mean(x^2) + eps) * (1 + weight)`` in fp32 over the last axis, then back to ``x.dtype``
+    (``transformers/models/gemma3/modeling_gemma3.py``, ``Gemma3RMSNorm.forward``)."""
+    xf = x.to(torch.float32)
+    normed = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    return (normed * (1.0 + weight.to(torch.float32))).to(x.dtype)
+
+
+def rope_closed_form(x, positions, max_wavelength: float = 10_000):
+    """Float64, element by element, through complex multiplication.  ``x`` nested lists / tensor
+    ``(B, L, H, D)``, ``positions (B, L)`` or ``(A, B, L)``.  Small inputs only."""
+    x = torch.as_tensor(x, dtype=torch.float64)
+    positions = torch.as_tensor(positions)
+    b_n, l_n, h_n, d = x.shape
+    half = d // 2
+    out = torch.empty_like(x)
+    for b in range(b_n):
+        for l in range(l_n):  # noqa: E741
+            for i in range(half):
+                if positions.ndim == 3:
+                    p = float(positions[i % positions.shape[0], b, l])
+                else:
+                    p = float(positions[b, l])
+                turn = cmath.exp(1j * p / float(max_wavelength) ** (2.0 * i / d))
+                for h in range(h_n):
+                    z = complex(float(x[b, l, h, i]), float(x[b, l, h, i + half])) * turn
+                    out[b, l, h, i], out[b, l, h, i + half] = z.real, z.imag
+    return out

@@ -1,0 +1,176 @@
+"""GPU parity of the rotary-embedding kernel against the oracle, through the C ABI.
+
+Bars: fp32 rel-L2 <= 1e-5; bf16 / fp16 rel-L2 <= 1e-2 and max-abs <= 2e-2 (and, tighter, at most a
+rounding step of the element type on a small share of the elements: both sides compute in fp32 and
+round once, so they differ only where sin / cos differ in their last bits)."""
+
+import pytest
+import torch
+
+from opentau_amd import rope as hip_rope
+from oracle import rope as oracle
+from tests.helpers import assert_close_bf16, max_abs, randn, rel_l2
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def g(t):
+    return t.to(DEV)
+
+
+def positions(b, length, seed, axes=0, hi=2000):
+    gen = torch.Generator().manual_seed(seed)
+    shape = (axes, b, length) if axes else (b, length)
+    return torch.randint(0, hi, shape, generator=gen)
+
+
+def check(got, want, dtype, what):
+    if dtype == torch.float32:
+        r = rel_l2(got, want)
+        assert r <= 1e-5, f"{what}: rel-L2 {r:.3e}"
+    else:
+        assert_close_bf16(got.float(), want.float(), what)
+        # one rounding step at most, on few elements
+        step = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+        diff = (got.double() - want.double()).abs()
+        assert float((diff / want.double().abs().clamp_min(1.0)).max()) <= 2 * step, what
+        assert float((diff > 0).double().mean()) <= 5e-3, what
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("b,length,h,hkv,d,axes", [
+    (2, 51, 8, 1, 256, 0),     # pi0.5 / PaliGemma head geometry
+    (1, 130, 16, 2, 128, 3),   # interleaved MRoPE over three axes
+    (3, 7, 5, 3, 64, 0),
+    (2, 33, 2, 2, 96, 2),      # head_dim that is no power of two
+    (1, 4, 1, 1, 32, 0),
+])
+def test_rope_qk_matches_oracle(dtype, b, length, h, hkv, d, axes):
+    q, k = randn((b, length, h, d), dtype, 1), randn((b, length, hkv, d), dtype, 2)
+    pos = positions(b, length, 3, axes)
+    for w in (10_000, 1_000_000):
+        qo, ko = hip_rope.apply_rope_qk(g(q), g(k), g(pos), w)
+        # the oracle on the same device computes the timescales with the ops the product uses
+        check(qo, oracle.apply_rope(g(q), g(pos), w), dtype, "q, oracle on the GPU")
+        check(ko, oracle.apply_rope(g(k), g(pos), w), dtype, "k, oracle on the GPU")
+    # the CPU oracle: its pow may round a timescale the other way, which moves an angle of ~2000 rad by ~1e-4
+    small = positions(b, length, 4, axes, hi=60)
+    qo, ko = hip_rope.apply_rope_qk(g(q), g(k), g(small))
+    check(qo.cpu(), oracle.apply_rope(q, small), dtype, "q, oracle on the CPU")
+    check(ko.cpu(), oracle.apply_rope(k, small), dtype, "k, oracle on the CPU")
+    single = hip_rope.apply_rope(g(q), g(small))
+    assert torch.equal(single, qo)
+
+
+def test_reference_cases_on_the_kernel():
+    # tests/policies/test_pi06.py:159-180 of the reference, run on the HIP path
+    x = g(randn((2, 4, 3, 32), torch.float32, 0))
+    pos = g(torch.arange(4)[None, :].expand(2, 4))
+    out = hip_rope.apply_rope(x, pos, max_wavelength=10_000.0)
+    assert out.shape == x.shape and out.dtype == x.dtype
+    assert not torch.allclose(out, hip_rope.apply_rope(x, pos, max_wavelength=1_000_000.0))
+    ones = torch.ones(1, 1, 1, 8, device=DEV)
+    assert torch.allclose(hip_rope.apply_rope(ones, torch.zeros(1, 1, dtype=torch.long, device=DEV)), ones, atol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_in_place_into_cache_rows_and_head_major_inputs(dtype):
+    b, length, h, hkv, d, n0 = 2, 50, 8, 1, 256, 712
+    pos = g(positions(b, length, 5))
+    # head-major storage (B, H, L, D) seen as (B, L, H, D): the kernel follows the strides
+    q_hm = g(randn((b, h, length, d), dtype, 1))
+    k = g(randn((b, length, hkv, d), dtype, 2))
+    want_q, want_k = hip_rope.apply_rope_qk(q_hm.transpose(1, 2).contiguous(), k, pos)
+    cache = torch.zeros(b, n0 + length, hkv, d, dtype=dtype, device=DEV)
+    q_view = q_hm.transpose(1, 2)
+    qo, ko = hip_rope.apply_rope_qk(q_view, k, pos, q_out=q_view, k_out=cache[:, n0:])
+    assert qo.data_ptr() == q_hm.data_ptr() and torch.equal(q_hm.transpose(1, 2), want_q)
+    assert torch.equal(cache[:, n0:], want_k) and not cache[:, :n0].any()
+    # one tensor at a time gives the same bits
+    assert torch.equal(hip_rope.rope_raw(None, k, pos)[1], want_k)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("b,length,h,hkv,d", [(2, 40, 8, 4, 256), (1, 19, 4, 1, 128), (2, 5, 2, 2, 32)])
+def test_fused_gemma3_norm_then_rope(dtype, b, length, h, hkv, d):
+    q, k = randn((b, length, h, d), dtype, 1) * 3.0, randn((b, length, hkv, d), dtype, 2) * 0.2
+    wq, wk = (randn((d,), torch.float32, 3) * 0.3).to(dtype), (randn((d,), torch.float32, 4) * 0.3).to(dtype)
+    pos = positions(b, length, 5)
+    qo, ko = hip_rope.apply_rope_qk(g(q), g(k), g(pos), 1_000_000, q_norm_weight=g(wq), k_norm_weight=g(wk),
+                                    norm_eps=1e-6)
+    want_q = oracle.apply_rope(oracle.gemma3_rms_norm(g(q), g(wq), 1e-6), g(pos), 1_000_000)
+    want_k = oracle.apply_rope(oracle.gemma3_rms_norm(g(k), g(wk), 1e-6), g(pos), 1_000_000)
+    if dtype == torch.float32:
+        assert rel_l2(qo, want_q) <= 1e-5 and rel_l2(ko, want_k) <= 1e-5
+    else:
+        # the norm is rounded to the element type before the rotation, on both sides; a row sum that
+        # differs in its last bit can move that rounding, which the rotation then carries along
+        assert_close_bf16(qo.float(), want_q.float(), "q")
+        assert_close_bf16(ko.float(), want_k.float(), "k")
+        assert rel_l2(qo.float(), want_q.float()) <= (2e-3 if dtype == torch.bfloat16 else 3e-4)
+    # norm on q only (pi0.6 norms the backbone stream only)
+    qo2, ko2 = hip_rope.apply_rope_qk(g(q), g(k), g(pos), 1_000_000, q_norm_weight=g(wq))
+    assert torch.equal(qo2, qo) and torch.equal(ko2, hip_rope.apply_rope(g(k), g(pos), 1_000_000))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_gradient_is_the_inverse_rotation(dtype):
+    b, length, h, hkv, d = 2, 23, 4, 2, 128
+    pos = positions(b, length, 6, hi=300)
+    q, k = randn((b, length, h, d), dtype, 1), randn((b, length, hkv, d), dtype, 2)
+    wq, wk = randn((b, length, h, d), dtype, 3), randn((b, length, hkv, d), dtype, 4)
+
+    def grads(fn, dev):
+        qq, kk = q.to(dev).requires_grad_(True), k.to(dev).requires_grad_(True)
+        qo, ko = fn(qq, kk, pos.to(dev))
+        ((qo.float() * wq.to(dev).float()).sum() + (ko.float() * wk.to(dev).float()).sum()).backward()
+        return qq.grad, kk.grad
+
+    got = grads(hip_rope.apply_rope_qk, DEV)
+    want = grads(lambda a, c, p: (oracle.apply_rope(a, p), oracle.apply_rope(c, p)), DEV)
+    for a, e, name in zip(got, want, ("dq", "dk")):
+        check(a, e, dtype, name)
+    if dtype == torch.float32:  # forward then inverse is the identity
+        y = hip_rope.rope_raw(g(q), None, g(pos))[0]
+        back = hip_rope.rope_raw(y, None, g(pos), inverse=True)[0]
+        assert max_abs(back.cpu(), q) <= 1e-5
+    single = q.to(DEV).requires_grad_(True)
+    (hip_rope.apply_rope(single, g(pos)).float() * g(wq).float()).sum().backward()
+    assert torch.equal(single.grad, got[0])
+
+
+def test_rope_full_training_shape_keeps_pair_norms():
+    """pi0.5 training shape (B32, S754, 8 + 1 heads of 256): a rotation keeps x[d]^2 + x[d + D/2]^2,
+    whatever the size; and the in-place call gives the same bits as the out-of-place one."""
+    b, length, h, hkv, d = 32, 754, 8, 1, 256
+    q, k = g(randn((b, length, h, d), torch.float32, 1)), g(randn((b, length, hkv, d), torch.float32, 2))
+    pos = g(torch.arange(length)[None, :].expand(b, length))
+    qo, ko = hip_rope.apply_rope_qk(q, k, pos)
+    n = lambda t: t[..., : d // 2] ** 2 + t[..., d // 2 :] ** 2  # noqa: E731
+    assert torch.allclose(n(qo), n(q), rtol=1e-5, atol=1e-6) and torch.allclose(n(ko), n(k), rtol=1e-5, atol=1e-6)
+    assert rel_l2(qo, oracle.apply_rope(q, pos)) <= 1e-5
+    qb, kb = q.bfloat16(), k.bfloat16()
+    want = hip_rope.apply_rope_qk(qb, kb, pos)
+    hip_rope.apply_rope_qk(qb, kb, pos, q_out=qb, k_out=kb)
+    assert torch.equal(qb, want[0]) and torch.equal(kb, want[1])
+
+
+def test_rope_argument_errors():
+    x = g(randn((1, 4, 2, 64), torch.bfloat16, 1))
+    pos = g(torch.zeros(1, 4, dtype=torch.long))
+    with pytest.raises(RuntimeError, match="head_dim"):
+        hip_rope.apply_rope(g(randn((1, 4, 2, 40), torch.bfloat16, 1)), pos)
+    with pytest.raises(RuntimeError, match="power-of-two"):
+        hip_rope.apply_rope_qk(g(randn((1, 4, 2, 96), torch.bfloat16, 1)), g(randn((1, 4, 2, 96), torch.bfloat16, 2)), pos,
+                               q_norm_weight=torch.zeros(96))
+    with pytest.raises(RuntimeError, match="positions"):
+        hip_rope.apply_rope(x, pos[:, :3])
+    with pytest.raises(RuntimeError, match="integers"):
+        hip_rope.apply_rope(x, pos.float())
+    with pytest.raises(RuntimeError, match="CPU"):
+        hip_rope.apply_rope(x.cpu(), pos.cpu())
+    with pytest.raises(RuntimeError, match="differ"):
+        hip_rope.apply_rope_qk(x, g(randn((1, 5, 2, 64), torch.bfloat16, 2)), pos)
+    with pytest.raises(RuntimeError, match="differentiable"):
+        hip_rope.apply_rope_qk(x.clone().requires_grad_(True), x, pos, q_out=torch.empty_like(x))
