@@ -364,6 +364,8 @@ int bcattn_rope(const bcattn_rope_params *p, void *stream) {
     return rc;
   if ((p->q.ptr && p->H <= 0) || (p->k.ptr && p->Hkv <= 0))
     return fail(BCATTN_ERR_INVALID, "bad head counts H=%d Hkv=%d", p->H, p->Hkv);
+  if ((p->q.ptr ? (int64_t)p->H : 0) + (p->k.ptr ? (int64_t)p->Hkv : 0) > 16384)
+    return fail(BCATTN_ERR_UNSUPPORTED, "more than 16384 heads");
   RopeArgs a;
   a.q = targ(p->q);
   a.k = targ(p->k);

@@ -2,12 +2,13 @@
 // front): an elementwise pass bound by HBM, read once and written once.
 //
 // A workgroup takes a few tokens.  Phase 1: one thread per (token, band) computes the sine
-// and cosine of that band's angle, once for all heads, into LDS.  Phase 2: the threads walk
-// over the (token, head, 16-byte piece) items; an item is a piece of the first half of a row
-// and the matching piece of the second half.  Consecutive lanes take consecutive pieces of a
-// row and then the next head, so with heads stored side by side a wave's loads and stores
-// cover one contiguous span.  The first items are requested before phase 1, so the trigonometry
-// runs under their latency.
+// and cosine of that band's angle, once for all heads, into LDS; one thread per token leaves
+// the token's element offsets in the four tensors there too.  Phase 2: the threads walk over
+// the (token, head, 16-byte piece) items; an item is a piece of the first half of a row and
+// the matching piece of the second half.  Consecutive lanes take consecutive pieces of a row
+// and then the next head, so with heads stored side by side a wave's loads and stores cover
+// one contiguous span.  The vector ALU is what competes with the memory system here, so the
+// index arithmetic avoids integer division and the trigonometry has a short path.
 #include "bcattn_common.h"
 
 namespace bcattn {
@@ -18,110 +19,152 @@ struct Vec {
 } __attribute__((aligned(16)));
 
 constexpr int kRopeThreads = 256;
-constexpr int kRopeUnroll = 2;  // items a thread has in flight
+constexpr int kRopeUnroll = 1;  // items a thread has in flight (measured: 2 is no faster, 4 is slower; occupancy does the overlapping)
 // Tokens per workgroup: enough for about this many items (measured: 600 to 1200 items per
 // workgroup run fastest at every shape tried; fewer leave the barrier and the trigonometry
 // exposed, more leave the last workgroups of a CU running alone), within 32 KB of LDS.
 constexpr int kRopeItems = 1024;
 inline int rope_tokens(int D, int items_per_token) {
   const int want = (kRopeItems + items_per_token / 2) / items_per_token;
-  const int fit = 8192 / D;
+  const int fit = 4096 / D;
   return want < 1 ? 1 : (want > fit ? fit : want);
 }
 
-template <typename T, int V>
-struct RopeItem {
-  const T *src;
-  T *dst;
-  const T *wgt;  // norm weights of the row's tensor, or null
-  int t;         // token slot in the workgroup
-  bool live;
-};
-
-template <typename T, int V>
-__device__ __forceinline__ RopeItem<T, V> rope_item(const RopeArgs &a, int item, int nitems, int tok0, int ntok,
-                                                    int lpr) {
-  // item = (token slot, row, piece), piece fastest; rows: the heads of q, then those of k
-  const int rows = (a.q.ptr ? a.H : 0) + (a.k.ptr ? a.Hkv : 0);
-  RopeItem<T, V> it;
-  const int c = item % lpr;
-  const int rest = item / lpr;
-  const int row = rest % rows;
-  it.t = rest / rows;
-  const int64_t tok = (int64_t)tok0 + it.t;
-  it.live = item < nitems && tok < ntok;
-  const int b = it.live ? (int)(tok / a.L) : 0, l = it.live ? (int)(tok % a.L) : 0;
-  const int nq = a.q.ptr ? a.H : 0;
-  const bool is_k = row >= nq;
-  const TensorArg &in = is_k ? a.k : a.q;
-  const TensorArg &out = is_k ? a.k_out : a.q_out;
-  const int h = is_k ? row - nq : row;
-  it.src = reinterpret_cast<const T *>(in.ptr) + b * in.sb + (int64_t)l * in.ss + h * in.sh + c * V;
-  it.dst = reinterpret_cast<T *>(const_cast<void *>(out.ptr)) + b * out.sb + (int64_t)l * out.ss + h * out.sh + c * V;
-  const void *w = is_k ? a.k_w : a.q_w;
-  it.wgt = w ? reinterpret_cast<const T *>(w) + c * V : nullptr;
-  return it;
+// floor(x / d) for 0 <= x < 2^22 and 0 < d < 2^22, with rcp = 1.0f / d: the float quotient is
+// off by one at most, which the remainder shows.
+__device__ __forceinline__ int small_div(int x, int d, float rcp) {
+  int q = (int)((float)x * rcp);
+  const int r = x - (int)__mul24(q, d);
+  q += r >= d ? 1 : 0;
+  q -= r < 0 ? 1 : 0;
+  return q;
 }
 
-template <typename T, int V>
-__global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeArgs a, const int TB) {
-#pragma clang fp contract(off)  // products and sums rounded one by one, as a framework's elementwise ops do
-  extern __shared__ __align__(16) float trig[];  // [tokens][half] sines, then as many cosines
+// sin and cos of an fp32 angle.  |x| < 3e4: reduction by multiples of pi/2 held in three
+// parts (each fma rounds once, the products are exact inside it), then the usual degree-7 /
+// degree-8 polynomials on [-pi/4, pi/4]; within two units in the last place.  Larger angles
+// take the library routine.
+__device__ __forceinline__ void rope_sincos(float x, float &sn, float &cs) {
+  if (!(fabsf(x) < 3.0e4f)) {
+    sincosf(x, &sn, &cs);
+    return;
+  }
+  const float kf = rintf(x * 0.63661977236758134308f);
+  float r = fmaf(kf, -1.57079625129699707031e+00f, x);
+  r = fmaf(kf, -7.54978941586159635335e-08f, r);
+  r = fmaf(kf, -5.39030285815811905290e-15f, r);
+  const int k = (int)kf;
+  const float z = r * r;
+  const float ps = fmaf(fmaf(fmaf(-1.9515295891e-4f, z, 8.3321608736e-3f), z, -1.6666654611e-1f), z * r, r);
+  const float pc = fmaf(fmaf(fmaf(2.443315711809948e-5f, z, -1.388731625493765e-3f), z, 4.166664568298827e-2f), z * z,
+                        fmaf(-0.5f, z, 1.0f));
+  const float s0 = (k & 1) ? pc : ps;
+  const float c0 = (k & 1) ? ps : pc;
+  sn = (k & 2) ? -s0 : s0;
+  cs = ((k + 1) & 2) ? -c0 : c0;
+}
+
+struct RopeToken {
+  int64_t q, k, q_out, k_out;  // element offsets of the token's first head in each tensor
+};
+
+// LPR: 16-byte pieces per row half when that is a power of two known at compile time, else 0
+// (read from the arguments).
+template <typename T, int V, int LPR>
+__global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeArgs a, const int TB, const float rcp_rows,
+                                                            const float rcp_lpr) {
+  extern __shared__ __align__(16) char rope_lds[];
   const int tid = threadIdx.x;
   const int half = a.D / 2;
-  const int lpr = half / V;  // lanes (pieces) per row
+  const int lpr = LPR ? LPR : half / V;
   const int ntok = a.B * a.L;
   const int tok0 = blockIdx.x * TB;
-  const int rows = (a.q.ptr ? a.H : 0) + (a.k.ptr ? a.Hkv : 0);
+  const int nq = a.q.ptr ? a.H : 0;
+  const int rows = nq + (a.k.ptr ? a.Hkv : 0);
   const int nitems = TB * rows * lpr;
-  float *sin_s = trig, *cos_s = trig + TB * half;
+  float *sin_s = reinterpret_cast<float *>(rope_lds), *cos_s = sin_s + TB * half;
+  RopeToken *tok_s = reinterpret_cast<RopeToken *>(cos_s + TB * half);
 
-  RopeItem<T, V> it[kRopeUnroll];
-  Vec<T, V> x1[kRopeUnroll], x2[kRopeUnroll];
-  auto request = [&](int first) __attribute__((always_inline)) {
-#pragma unroll
-    for (int u = 0; u < kRopeUnroll; ++u) {
-      it[u] = rope_item<T, V>(a, first + u * kRopeThreads, nitems, tok0, ntok, lpr);
-      if (it[u].live) {
-        x1[u] = *reinterpret_cast<const Vec<T, V> *>(it[u].src);
-        x2[u] = *reinterpret_cast<const Vec<T, V> *>(it[u].src + half);
-      }
-    }
+  // ---- phase 1 ----------------------------------------------------------------------------
+  const int b0 = tok0 / a.L, l0 = tok0 - b0 * a.L;  // uniform
+  auto batch_pos = [&](int t, int &b, int &l) __attribute__((always_inline)) {
+    b = b0, l = l0 + t;
+    if (l >= a.L) b += l / a.L, l %= a.L;  // only workgroups that straddle samples get here
   };
-  request(tid);
-
-  // ---- phase 1: one (token, band) pair per thread and step ----------------------------------
+  const float rcp_half = 1.0f / (float)half;
   for (int p = tid; p < TB * half; p += kRopeThreads) {
-    const int t = p / half, band = p % half;
-    const int64_t tok = (int64_t)tok0 + t;
+    const int t = small_div(p, half, rcp_half), band = p - t * half;
     float sn = 0.f, cs = 1.f;
-    if (tok < ntok) {
-      const int b = (int)(tok / a.L), l = (int)(tok % a.L);
+    if (tok0 + t < ntok) {
+      int b, l;
+      batch_pos(t, b, l);
       const int axis = a.n_axes > 1 ? band % a.n_axes : 0;
       const float pos = (float)a.positions[((int64_t)axis * a.B + b) * a.L + l];
-      const float ang = __fdiv_rn(pos, a.timescale[band]);
-      sincosf(ang, &sn, &cs);
+      rope_sincos(__fdiv_rn(pos, a.timescale[band]), sn, cs);
       if (a.inverse) sn = -sn;
     }
     sin_s[p] = sn;
     cos_s[p] = cs;
   }
-  // LDS writes done, then the barrier; the requested rows stay in flight across it
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  for (int t = tid; t < TB; t += kRopeThreads) {
+    int b, l;
+    batch_pos(t, b, l);
+    if (tok0 + t >= ntok) b = l = 0;
+    RopeToken o;
+    o.q = b * a.q.sb + (int64_t)l * a.q.ss;
+    o.k = b * a.k.sb + (int64_t)l * a.k.ss;
+    o.q_out = b * a.q_out.sb + (int64_t)l * a.q_out.ss;
+    o.k_out = b * a.k_out.sb + (int64_t)l * a.k_out.ss;
+    tok_s[t] = o;
+  }
+  __syncthreads();
 
-  // ---- phase 2 --------------------------------------------------------------------------------
+  // ---- phase 2 ----------------------------------------------------------------------------
   for (int first = tid; first < nitems; first += kRopeUnroll * kRopeThreads) {
-    if (first != tid) request(first);
+#pragma clang fp contract(off)  // products and sums rounded one by one, as a framework's elementwise ops do
+    const T *src[kRopeUnroll];
+    T *dst[kRopeUnroll];
+    const T *wgt[kRopeUnroll];
+    int trig[kRopeUnroll];  // index of the item's first sine / cosine
+    bool live[kRopeUnroll];
+    Vec<T, V> x1[kRopeUnroll], x2[kRopeUnroll];
 #pragma unroll
     for (int u = 0; u < kRopeUnroll; ++u) {
-      if (!it[u].live) continue;
+      // item = (token slot, row, piece), piece fastest; rows: the heads of q, then those of k
+      const int item = first + u * kRopeThreads;
+      int c, rest;
+      if (LPR) {
+        c = item & (LPR - 1), rest = item / (LPR ? LPR : 1);
+      } else {
+        rest = small_div(item, lpr, rcp_lpr), c = item - rest * lpr;
+      }
+      const int t = small_div(rest, rows, rcp_rows), row = rest - t * rows;
+      live[u] = item < nitems && tok0 + t < ntok;
+      const RopeToken o = tok_s[live[u] ? t : 0];
+      const bool is_k = row >= nq;
+      const int h = is_k ? row - nq : row;
+      const int64_t sh_in = is_k ? a.k.sh : a.q.sh, sh_out = is_k ? a.k_out.sh : a.q_out.sh;
+      src[u] = reinterpret_cast<const T *>(is_k ? a.k.ptr : a.q.ptr) + (is_k ? o.k : o.q) + h * sh_in + c * V;
+      dst[u] = reinterpret_cast<T *>(const_cast<void *>(is_k ? a.k_out.ptr : a.q_out.ptr)) +
+               (is_k ? o.k_out : o.q_out) + h * sh_out + c * V;
+      const void *w = is_k ? a.k_w : a.q_w;
+      wgt[u] = w ? reinterpret_cast<const T *>(w) + c * V : nullptr;
+      trig[u] = t * half + c * V;
+      if (live[u]) {
+        x1[u] = *reinterpret_cast<const Vec<T, V> *>(src[u]);
+        x2[u] = *reinterpret_cast<const Vec<T, V> *>(src[u] + half);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kRopeUnroll; ++u) {
+      if (!live[u]) continue;
       float f1[V], f2[V];
 #pragma unroll
       for (int e = 0; e < V; ++e) {
         f1[e] = (float)x1[u].v[e];
         f2[e] = (float)x2[u].v[e];
       }
-      if (it[u].wgt != nullptr) {
+      if (wgt[u] != nullptr) {
         // The lpr lanes of a row are neighbours, aligned to lpr (a power of two here), and take
         // this branch together.
         float ss = 0.f;
@@ -129,16 +172,15 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeArgs a, co
         for (int e = 0; e < V; ++e) ss += f1[e] * f1[e] + f2[e] * f2[e];
         for (int o = 1; o < lpr; o <<= 1) ss += __shfl_xor(ss, o, 64);
         const float r = 1.0f / sqrtf(ss / (float)a.D + a.eps);
-        const Vec<T, V> w1 = *reinterpret_cast<const Vec<T, V> *>(it[u].wgt);
-        const Vec<T, V> w2 = *reinterpret_cast<const Vec<T, V> *>(it[u].wgt + half);
+        const Vec<T, V> w1 = *reinterpret_cast<const Vec<T, V> *>(wgt[u]);
+        const Vec<T, V> w2 = *reinterpret_cast<const Vec<T, V> *>(wgt[u] + half);
 #pragma unroll
         for (int e = 0; e < V; ++e) {  // rounded to the element type, as the norm module returns it
           f1[e] = (float)(T)((f1[e] * r) * (1.0f + (float)w1.v[e]));
           f2[e] = (float)(T)((f2[e] * r) * (1.0f + (float)w2.v[e]));
         }
       }
-      const int c = (first + u * kRopeThreads) % lpr;
-      const float *sp = sin_s + it[u].t * half + c * V, *cp = cos_s + it[u].t * half + c * V;
+      const float *sp = sin_s + trig[u], *cp = cos_s + trig[u];
       Vec<T, V> y1, y2;
 #pragma unroll
       for (int e = 0; e < V; ++e) {
@@ -146,25 +188,38 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeArgs a, co
         y1.v[e] = (T)(f1[e] * cs - f2[e] * sn);
         y2.v[e] = (T)(f2[e] * cs + f1[e] * sn);
       }
-      *reinterpret_cast<Vec<T, V> *>(it[u].dst) = y1;
-      *reinterpret_cast<Vec<T, V> *>(it[u].dst + half) = y2;
+      *reinterpret_cast<Vec<T, V> *>(dst[u]) = y1;
+      *reinterpret_cast<Vec<T, V> *>(dst[u] + half) = y2;
     }
   }
 }
 
-int launch_rope(const RopeArgs &a, int dtype, hipStream_t st) {
+template <typename T, int V>
+static void launch_rope_t(const RopeArgs &a, int rows, hipStream_t st) {
+  const int lpr = a.D / (2 * V);
+  const int TB = rope_tokens(a.D, rows * lpr);
   const int64_t ntok = (int64_t)a.B * a.L;
-  const int rows = (a.q.ptr ? a.H : 0) + (a.k.ptr ? a.Hkv : 0);
-  if (ntok == 0 || rows == 0) return BCATTN_OK;
-  const int TB = rope_tokens(a.D, rows * (a.D / (dtype == BCATTN_F32 ? 8 : 16)));
   const dim3 grid((unsigned)((ntok + TB - 1) / TB)), block(kRopeThreads);
-  const size_t lds = (size_t)TB * a.D * sizeof(float);
+  const size_t lds = (size_t)TB * a.D * sizeof(float) + (size_t)TB * sizeof(RopeToken);
+  const float rr = 1.0f / (float)rows, rl = 1.0f / (float)lpr;
+  switch (lpr) {
+    case 4: hipLaunchKernelGGL((rope_kernel<T, V, 4>), grid, block, lds, st, a, TB, rr, rl); break;
+    case 8: hipLaunchKernelGGL((rope_kernel<T, V, 8>), grid, block, lds, st, a, TB, rr, rl); break;
+    case 16: hipLaunchKernelGGL((rope_kernel<T, V, 16>), grid, block, lds, st, a, TB, rr, rl); break;
+    case 32: hipLaunchKernelGGL((rope_kernel<T, V, 32>), grid, block, lds, st, a, TB, rr, rl); break;
+    default: hipLaunchKernelGGL((rope_kernel<T, V, 0>), grid, block, lds, st, a, TB, rr, rl); break;
+  }
+}
+
+int launch_rope(const RopeArgs &a, int dtype, hipStream_t st) {
+  const int rows = (a.q.ptr ? a.H : 0) + (a.k.ptr ? a.Hkv : 0);
+  if ((int64_t)a.B * a.L == 0 || rows == 0) return BCATTN_OK;
   if (dtype == BCATTN_F32)
-    hipLaunchKernelGGL((rope_kernel<float, 4>), grid, block, lds, st, a, TB);
+    launch_rope_t<float, 4>(a, rows, st);
   else if (dtype == BCATTN_BF16)
-    hipLaunchKernelGGL((rope_kernel<__bf16, 8>), grid, block, lds, st, a, TB);
+    launch_rope_t<__bf16, 8>(a, rows, st);
   else
-    hipLaunchKernelGGL((rope_kernel<_Float16, 8>), grid, block, lds, st, a, TB);
+    launch_rope_t<_Float16, 8>(a, rows, st);
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
 }
 
