@@ -1070,7 +1070,7 @@ static int launch_dkv(const BwdArgs &a, hipStream_t st) {
 
 // The dQ and the dK/dV kernels are independent, and each leaves part of the chip idle
 // while its last workgroups finish (a workgroup holds most of a CU's LDS, so the grid is
-// a small number of "rounds").  When a call runs both, the dK/dV kernel goes to a side
+// a small number of "rounds").  When a call runs both, one of them goes to a side
 // stream that is forked from and joined to the caller's stream by events, and the two
 // kernels' workgroups share the chip.  One side stream and event pair per device, made
 // on first use and kept; default priority; calls on one device take turns using them.
@@ -1116,7 +1116,7 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
   const bool both = (a.stages & BCATTN_BWD_DQ) && (a.stages & BCATTN_BWD_DKV);
   SideStream *ss = both ? side_stream() : nullptr;
   std::unique_lock<std::mutex> turn;
-  hipStream_t kst = st;  // stream of the dK/dV kernel
+  hipStream_t kst = st;  // the other stream, when there is one
   if (ss) {
     turn = std::unique_lock<std::mutex>(ss->mu);
     if (hipEventRecord(ss->fork, st) == hipSuccess && hipStreamWaitEvent(ss->stream, ss->fork, 0) == hipSuccess)
@@ -1125,13 +1125,20 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
       ss = nullptr;
   }
   int rc = BCATTN_OK;
+  // Work on the helper stream starts a little later than work on the caller's stream (it waits
+  // for the fork event).  A dK/dV grid that cannot fill the chip by itself goes first, on the
+  // caller's stream, and the dQ workgroups fill the CUs it leaves (4 % on the pi0.5 training
+  // shape); a larger one goes to the helper stream (1 % better on the others).
+  constexpr int kKeysPerGroup = 32 * (PAIRS > 0 ? PAIRS : NWK);
+  const bool dkv_first = (int64_t)((a.Sk + kKeysPerGroup - 1) / kKeysPerGroup) * a.Hkv * a.B < kSplitTarget;
+  const hipStream_t dkv_st = dkv_first ? st : kst, dq_st = dkv_first ? kst : st;
   if (a.stages & BCATTN_BWD_DKV) {
     if constexpr (PAIRS > 0) {
-      rc = launch_dkv_pair<D, PAIRS>(a, kst);
+      rc = launch_dkv_pair<D, PAIRS>(a, dkv_st);
     } else if constexpr (SPLIT) {
-      if (!(rc = launch_dkv<D, NWK, kModeDV>(a, kst))) rc = launch_dkv<D, NWK, kModeDK>(a, kst);
+      if (!(rc = launch_dkv<D, NWK, kModeDV>(a, dkv_st))) rc = launch_dkv<D, NWK, kModeDK>(a, dkv_st);
     } else {
-      rc = launch_dkv<D, NWK, kModeBoth>(a, kst);
+      rc = launch_dkv<D, NWK, kModeBoth>(a, dkv_st);
     }
   }
   if (!rc && (a.stages & BCATTN_BWD_DQ)) {
@@ -1139,7 +1146,7 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
     const int ntile_r = (R + 32 * NWQ - 1) / (32 * NWQ);
     const size_t smem = dq_smem_bytes<D>() + needed_table_bytes((a.Sk + 63) / 64);
     hipLaunchKernelGGL((bwd_dq_kernel<D, NWQ>), dim3(xcd_grid((unsigned)(ntile_r * a.Hkv * a.B))), dim3(64 * NWQ),
-                       smem, st, a);
+                       smem, dq_st, a);
   }
   if (ss) {  // join, whatever happened in between: the caller's stream must not run ahead of the side stream
     if (hipEventRecord(ss->join, ss->stream) != hipSuccess || hipStreamWaitEvent(st, ss->join, 0) != hipSuccess)
