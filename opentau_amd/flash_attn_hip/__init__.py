@@ -240,6 +240,16 @@ def forward_raw(
     return out, lse
 
 
+def kvcache_workspace_bytes(b: int, sq: int, sk0: int, sk1: int, h: int, hkv: int, d: int,
+                            dtype: torch.dtype = torch.bfloat16) -> int:
+    """Bytes of workspace the KV-cached call needs at these sizes (``bcattn_fwd_kvcache_workspace_bytes``)."""
+    lib = _loader.require_library()
+    p = _loader.FwdParams()
+    p.B, p.Sq, p.Sk0, p.Sk1, p.H, p.Hkv, p.D = b, sq, sk0, sk1, h, hkv, d
+    p.dtype = _DTYPES[dtype][0]
+    return int(lib.bcattn_fwd_kvcache_workspace_bytes(ctypes.byref(p)))
+
+
 def backward_raw(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale: float, *, stages: int = 0,
                  workspace: torch.Tensor | None = None, summary_ready: bool = False, grads=None):
     """One backward through the C ABI.  Returns ``(dq, dk, dv)``.
