@@ -116,25 +116,52 @@ def rope_raw(
     return (q_out if q is not None else None), (k_out if k is not None else None)
 
 
-class _Rope(torch.autograd.Function):
-    """The rotation is orthogonal: its gradient is the rotation by minus the angle."""
+# The differentiable / traceable forms are torch.library ops (like the attention calls), so that
+# ``torch.compile`` traces through them with the fake implementations and autograd sees the
+# registered backward.  The rotation is orthogonal: its gradient is the rotation by minus the angle.
+@torch.library.custom_op("bcattn::rope", mutates_args=())
+def _op_rope(x: torch.Tensor, positions: torch.Tensor, max_wavelength: float, inverse: bool) -> torch.Tensor:
+    return rope_raw(x, None, positions, max_wavelength, inverse=inverse)[0]
 
-    @staticmethod
-    def forward(ctx, q, k, positions, max_wavelength):
-        ctx.save_for_backward(positions)
-        ctx.max_wavelength = max_wavelength
-        ctx.has = (q is not None, k is not None)
-        qo, ko = rope_raw(q, k, positions, max_wavelength)
-        return tuple(t for t in (qo, ko) if t is not None)
 
-    @staticmethod
-    def backward(ctx, *grads):
-        (positions,) = ctx.saved_tensors
-        it = iter(grads)
-        gq = next(it).contiguous() if ctx.has[0] else None
-        gk = next(it).contiguous() if ctx.has[1] else None
-        dq, dk = rope_raw(gq, gk, positions, ctx.max_wavelength, inverse=True)
-        return dq, dk, None, None
+@_op_rope.register_fake
+def _(x, positions, max_wavelength, inverse):
+    return x.new_empty(x.shape)
+
+
+@torch.library.custom_op("bcattn::rope_qk", mutates_args=())
+def _op_rope_qk(q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor, max_wavelength: float,
+                inverse: bool) -> tuple[torch.Tensor, torch.Tensor]:
+    return rope_raw(q, k, positions, max_wavelength, inverse=inverse)
+
+
+@_op_rope_qk.register_fake
+def _(q, k, positions, max_wavelength, inverse):
+    return q.new_empty(q.shape), k.new_empty(k.shape)
+
+
+def _rope_setup(ctx, inputs, output):
+    ctx.save_for_backward(inputs[-3])
+    ctx.max_wavelength, ctx.inverse = inputs[-2], inputs[-1]
+
+
+def _rope_backward(ctx, grad):
+    (positions,) = ctx.saved_tensors
+    return _op_rope(grad.contiguous(), positions, ctx.max_wavelength, not ctx.inverse), None, None, None
+
+
+def _rope_qk_backward(ctx, grad_q, grad_k):
+    (positions,) = ctx.saved_tensors
+    dq, dk = _op_rope_qk(grad_q.contiguous(), grad_k.contiguous(), positions, ctx.max_wavelength, not ctx.inverse)
+    return dq, dk, None, None, None
+
+
+_op_rope.register_autograd(_rope_backward, setup_context=_rope_setup)
+_op_rope_qk.register_autograd(_rope_qk_backward, setup_context=_rope_setup)
+
+
+def _needs_graph(*ts: torch.Tensor) -> bool:
+    return torch.compiler.is_compiling() or (torch.is_grad_enabled() and any(t.requires_grad for t in ts))
 
 
 def apply_rope(x: torch.Tensor, positions: torch.Tensor, max_wavelength: float = 10_000) -> torch.Tensor:
@@ -144,8 +171,8 @@ def apply_rope(x: torch.Tensor, positions: torch.Tensor, max_wavelength: float =
     fp32 arithmetic, one rounding to ``x.dtype``; with 3-D positions band ``i`` follows axis
     ``i % A`` (interleaved MRoPE).  Differentiable in ``x``.
     """
-    if torch.is_grad_enabled() and x.requires_grad:
-        return _Rope.apply(x, None, positions, max_wavelength)[0]
+    if _needs_graph(x):
+        return _op_rope(x, positions, float(max_wavelength), False)
     return rope_raw(x, None, positions, max_wavelength)[0]
 
 
@@ -170,9 +197,9 @@ def apply_rope_qk(
     other storage, e.g. ``cache_k[:, n0:n0 + L]`` of a preallocated key cache.
     """
     norm = q_norm_weight is not None or k_norm_weight is not None
-    if torch.is_grad_enabled() and (q.requires_grad or k.requires_grad):
+    if _needs_graph(q, k):
         if norm or q_out is not None or k_out is not None:
-            raise RuntimeError("apply_rope_qk is differentiable only without norm weights and output arguments")
-        return _Rope.apply(q, k, positions, max_wavelength)
+            raise RuntimeError("apply_rope_qk is differentiable / traceable only without norm weights and output arguments")
+        return _op_rope_qk(q, k, positions, float(max_wavelength), False)
     return rope_raw(q, k, positions, max_wavelength, q_out=q_out, k_out=k_out, q_norm_weight=q_norm_weight,
                     k_norm_weight=k_norm_weight, norm_eps=norm_eps)

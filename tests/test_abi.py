@@ -142,6 +142,12 @@ def test_fake_impl_gives_shapes_without_running_kernels():
         assert lse.shape == (2, 8, 50) and lse.dtype == torch.float32
         dq, dk, dv = torch.ops.bcattn.bwd(out, q, k, k, out, lse, *ids, 0.0625)
         assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == k.shape
+        import opentau_amd.rope  # noqa: F401  (registers the rotary ops)
+
+        pos = torch.empty(2, 50, dtype=torch.long)
+        rq, rk = torch.ops.bcattn.rope_qk(q, k[:, :50], pos, 10000.0, False)
+        assert rq.shape == q.shape and rk.shape == (2, 50, 1, 256) and rk.dtype == torch.bfloat16
+        assert torch.ops.bcattn.rope(q, pos, 10000.0, True).shape == q.shape
 
 
 def test_workloads_are_seeded_and_shaped():

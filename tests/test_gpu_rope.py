@@ -140,6 +140,28 @@ def test_rope_gradient_is_the_inverse_rotation(dtype):
     assert torch.equal(single.grad, got[0])
 
 
+def test_rope_traces_under_torch_compile():
+    """``torch.compile`` (backend ``aot_eager``: captured and replayed, nothing generated) goes through the
+    registered ops, forward and backward, and gives the eager bits."""
+    b, length, h, hkv, d = 2, 19, 4, 2, 64
+    pos = g(positions(b, length, 7, hi=500))
+    q0, k0 = g(randn((b, length, h, d), torch.bfloat16, 1)), g(randn((b, length, hkv, d), torch.bfloat16, 2))
+    wq, wk = g(randn((b, length, h, d), torch.bfloat16, 3)), g(randn((b, length, hkv, d), torch.bfloat16, 4))
+
+    def fn(q, k):
+        qo, ko = hip_rope.apply_rope_qk(q * 1.0, k, pos)
+        return qo, hip_rope.apply_rope(ko, pos, 1_000_000)
+
+    def run(f):
+        q, k = q0.clone().requires_grad_(True), k0.clone().requires_grad_(True)
+        qo, ko = f(q, k)
+        ((qo.float() * wq.float()).sum() + (ko.float() * wk.float()).sum()).backward()
+        return qo.detach(), ko.detach(), q.grad, k.grad
+
+    for a, c in zip(run(fn), run(torch.compile(fn, backend="aot_eager", fullgraph=True))):
+        assert torch.equal(a, c)
+
+
 def test_rope_full_training_shape_keeps_pair_norms():
     """pi0.5 training shape (B32, S754, 8 + 1 heads of 256): a rotation keeps x[d]^2 + x[d + D/2]^2,
     whatever the size; and the in-place call gives the same bits as the out-of-place one."""
