@@ -59,6 +59,11 @@ class StaticKVCache:
         self.length = n
         return k_rows, v_rows
 
+    def reset(self) -> None:
+        """Forget the rows and the mask summary (a new observation; or block ids that were changed in place)."""
+        self.length = 0
+        self._ids = None
+
     def layer(self, layer: int) -> tuple[torch.Tensor, torch.Tensor]:
         """The valid rows of a layer, ``(B, length, Hkv, D)`` views."""
         return self.k[layer, :, : self.length], self.v[layer, :, : self.length]

@@ -56,6 +56,7 @@ def _positions(positions: torch.Tensor, b: int, length: int) -> tuple[torch.Tens
         raise RuntimeError(f"positions {tuple(positions.shape)} do not match (B, L) = {(b, length)}")
     if positions.is_floating_point():
         raise RuntimeError("positions must be integers")
+    # (the kernel reads int32: positions are token indices, far below 2^31)
     return positions.to(torch.int32).contiguous(), n_axes
 
 
