@@ -24,8 +24,38 @@ def _expected(name):
         return {k: torch.from_numpy(z[k]) for k in ("out", "lse", "dq", "dk", "dv")}
 
 
+ROPE_NAMES = sorted(fixtures.ROPE_CASES)
+
+
 def test_every_case_has_its_fixture():
-    assert sorted(p.stem for p in GOLDEN.glob("*.npz")) == NAMES
+    assert sorted(p.stem for p in GOLDEN.glob("*.npz")) == sorted(NAMES + ROPE_NAMES)
+
+
+def _rope_expected(name):
+    with np.load(GOLDEN / f"{name}.npz") as z:
+        return torch.from_numpy(z["out"])
+
+
+@pytest.mark.parametrize("name", ROPE_NAMES)
+def test_rope_oracle_reproduces_the_fixtures(name):
+    from oracle import rope as oracle_rope
+
+    x, positions, w = fixtures.rope_inputs(name)
+    assert rel_l2(oracle_rope.apply_rope(x, positions, w), _rope_expected(name)) <= 1e-6
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,rel", [(torch.float32, 1e-5), (torch.bfloat16, 1e-2), (torch.float16, 2e-3)])
+@pytest.mark.parametrize("name", ROPE_NAMES)
+def test_rope_kernel_reproduces_the_fixtures(name, dtype, rel):
+    from opentau_amd import rope as hip_rope
+    from oracle import rope as oracle_rope
+
+    x, positions, w = fixtures.rope_inputs(name, dtype)
+    # a 16-bit run is held to the closed form on the rounded inputs
+    want = _rope_expected(name) if dtype == torch.float32 else oracle_rope.rope_closed_form(x.float(), positions, w)
+    got = hip_rope.apply_rope(x.to("cuda:0"), positions.to("cuda:0"), w)
+    assert got.dtype == dtype and rel_l2(got.float().cpu(), want) <= rel
 
 
 @pytest.mark.parametrize("name", NAMES)
