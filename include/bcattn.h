@@ -52,7 +52,7 @@
 extern "C" {
 #endif
 
-#define BCATTN_ABI_VERSION 2
+#define BCATTN_ABI_VERSION 3
 
 enum bcattn_dtype { BCATTN_F32 = 0, BCATTN_BF16 = 1, BCATTN_F16 = 2 };
 
@@ -189,8 +189,21 @@ int bcattn_bwd(const bcattn_bwd_params *p, void *stream);
  * in fp32, rounded once to the element type, as the reference does.  The caller
  * supplies the D/2 timescales (so they are the very numbers its framework
  * computes).  With n_axes > 1 (interleaved MRoPE) band d reads the position of
- * axis d % n_axes.  The norm, when asked for, is Gemma-3's: x * rsqrt(mean(x^2) +
- * eps) * (1 + w), rounded to the element type before the rotation.
+ * axis d % n_axes.
+ *
+ * Second form, when cos / sin tables are given: the rotation as cosmos3's expert
+ * applies it (src/opentau/policies/cosmos3/qwen3vl_with_expert.py:224, which calls
+ * transformers' apply_rotary_pos_emb with the backbone's (cos, sin)):
+ *     out = x * cos + rotate_half(x) * sin,   rotate_half(x) = (-x[D/2:], x[:D/2])
+ * with cos, sin (B, L, D) in the element type of the call and every product and
+ * sum rounded to that type, as elementwise framework ops in that type do.
+ * positions and timescale are not read then.
+ *
+ * The norm in front, when weights are given (fp32, D values; a 16-bit module
+ * weight converts exactly): BCATTN_NORM_GEMMA3  x * rsqrt(mean(x^2) + eps) * (1 + w)
+ * rounded to the element type (Gemma3RMSNorm, pi06/gemma3_with_expert.py:851-861);
+ * BCATTN_NORM_QWEN3  w * (x * rsqrt(mean(x^2) + eps) rounded to the element type),
+ * rounded again (ExpertRMSNorm, cosmos3/qwen3vl_with_expert.py:85-102, :217-218).
  *
  * An output may be its input (in place), or any other strided tensor: e.g. the
  * rows of a preallocated key cache that this layer's keys belong in.
@@ -202,14 +215,18 @@ typedef struct bcattn_rope_params {
   bcattn_tensor q_out, k_out; /* same shapes, out */
   const int32_t *positions;   /* (n_axes, B, L) contiguous */
   const float *timescale;     /* (D/2) */
-  const void *q_norm_weight;  /* (D) in the element type of the call, or null: no norm on q */
-  const void *k_norm_weight;  /* likewise for k */
+  const void *cos, *sin;      /* (B, L, D) contiguous, element type of the call; both null: angles from positions */
+  const float *q_norm_weight; /* (D) or null: no norm on q */
+  const float *k_norm_weight; /* likewise for k */
   int32_t B, L, H, Hkv, D;
   int32_t n_axes;
   int32_t dtype;              /* enum bcattn_dtype */
-  int32_t inverse;            /* nonzero: turn by minus the angle, which maps an output gradient to the input gradient; no norm then */
+  int32_t inverse;            /* nonzero: the map from an output gradient to the input gradient (the turn by minus the angle); no norm then */
+  int32_t norm_kind;          /* enum bcattn_norm_kind */
   float norm_eps;
 } bcattn_rope_params;
+
+enum bcattn_norm_kind { BCATTN_NORM_GEMMA3 = 0, BCATTN_NORM_QWEN3 = 1 };
 
 int bcattn_rope(const bcattn_rope_params *p, void *stream);
 

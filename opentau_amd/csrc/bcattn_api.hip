@@ -347,16 +347,18 @@ int bcattn_rope(const bcattn_rope_params *p, void *stream) {
   if ((int64_t)p->B * p->L >= ((int64_t)1 << 31) - 64) return fail(BCATTN_ERR_UNSUPPORTED, "B*L too large");
   if (p->D % (2 * vec) || p->D > 512)
     return fail(BCATTN_ERR_UNSUPPORTED, "rope needs head_dim %% %d == 0 and <= 512; got %d", 2 * vec, p->D);
-  if (p->positions == nullptr || p->timescale == nullptr)
+  const bool tables = p->cos != nullptr || p->sin != nullptr;
+  if (tables && (p->cos == nullptr || p->sin == nullptr))
+    return fail(BCATTN_ERR_INVALID, "cos and sin tables come together");
+  if (!tables && (p->positions == nullptr || p->timescale == nullptr))
     return fail(BCATTN_ERR_INVALID, "null positions / timescale pointer");
-  if (!aligned16(p->timescale)) return fail(BCATTN_ERR_INVALID, "timescale: pointer not 16-byte aligned");
+  if (p->norm_kind != BCATTN_NORM_GEMMA3 && p->norm_kind != BCATTN_NORM_QWEN3)
+    return fail(BCATTN_ERR_INVALID, "norm_kind %d unknown", p->norm_kind);
   const bool norm = p->q_norm_weight != nullptr || p->k_norm_weight != nullptr;
   if (norm && (p->D & (p->D - 1)))
     return fail(BCATTN_ERR_UNSUPPORTED, "the fused norm needs a power-of-two head_dim; got %d", p->D);
   if (norm && p->inverse) return fail(BCATTN_ERR_INVALID, "inverse rotation takes no norm");
   if (norm && !(p->norm_eps >= 0.f)) return fail(BCATTN_ERR_INVALID, "norm_eps must be non-negative");
-  if ((p->q_norm_weight && !aligned16(p->q_norm_weight)) || (p->k_norm_weight && !aligned16(p->k_norm_weight)))
-    return fail(BCATTN_ERR_INVALID, "norm weight: pointer not 16-byte aligned");
   int rc;
   if ((rc = check_tensor("q", p->q, vec, false)) || (rc = check_tensor("k", p->k, vec, false))) return rc;
   if ((rc = check_tensor("q_out", p->q_out, vec, p->q.ptr != nullptr)) ||
@@ -373,6 +375,9 @@ int bcattn_rope(const bcattn_rope_params *p, void *stream) {
   a.k_out = targ(p->k_out);
   a.positions = p->positions;
   a.timescale = p->timescale;
+  a.cos_t = p->cos;
+  a.sin_t = p->sin;
+  a.norm_kind = p->norm_kind;
   a.q_w = p->q.ptr ? p->q_norm_weight : nullptr;
   a.k_w = p->k.ptr ? p->k_norm_weight : nullptr;
   a.B = p->B;

@@ -158,8 +158,9 @@ struct RopeArgs {
   TensorArg q, k, q_out, k_out;  // a null ptr skips the tensor
   const int32_t *positions;      // (n_axes, B, L)
   const float *timescale;        // (D/2)
-  const void *q_w, *k_w;         // norm weights (D) or null
-  int B, L, H, Hkv, D, n_axes, inverse;
+  const void *cos_t, *sin_t;     // (B, L, D) tables in the element type, or null: angles from positions
+  const float *q_w, *k_w;        // norm weights (D) or null
+  int B, L, H, Hkv, D, n_axes, inverse, norm_kind;
   float eps;
 };
 int launch_rope(const RopeArgs &a, int dtype, hipStream_t st);

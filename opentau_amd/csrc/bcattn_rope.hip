@@ -70,7 +70,11 @@ struct RopeToken {
 
 // LPR: 16-byte pieces per row half when that is a power of two known at compile time, else 0
 // (read from the arguments).
-template <typename T, int V, int LPR>
+// TABLES: the cosines and sines come as (B, L, D) tables in the element type and every product
+// and sum is rounded to the element type (the form of a framework that rotates in the tensors'
+// own type: q * cos + rotate_half(q) * sin); otherwise they are computed here from positions and
+// the arithmetic is fp32 with one rounding at the end.
+template <typename T, int V, int LPR, bool TABLES>
 __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeArgs a, const int TB, const float rcp_rows,
                                                             const float rcp_lpr) {
   extern __shared__ __align__(16) char rope_lds[];
@@ -82,8 +86,9 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeArgs a, co
   const int nq = a.q.ptr ? a.H : 0;
   const int rows = nq + (a.k.ptr ? a.Hkv : 0);
   const int nitems = TB * rows * lpr;
-  float *sin_s = reinterpret_cast<float *>(rope_lds), *cos_s = sin_s + TB * half;
-  RopeToken *tok_s = reinterpret_cast<RopeToken *>(cos_s + TB * half);
+  const int TW = TABLES ? a.D : half;  // sines (cosines) kept per token
+  float *sin_s = reinterpret_cast<float *>(rope_lds), *cos_s = sin_s + TB * TW;
+  RopeToken *tok_s = reinterpret_cast<RopeToken *>(cos_s + TB * TW);
 
   // ---- phase 1 ----------------------------------------------------------------------------
   const int b0 = tok0 / a.L, l0 = tok0 - b0 * a.L;  // uniform
@@ -91,17 +96,23 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeArgs a, co
     b = b0, l = l0 + t;
     if (l >= a.L) b += l / a.L, l %= a.L;  // only workgroups that straddle samples get here
   };
-  const float rcp_half = 1.0f / (float)half;
-  for (int p = tid; p < TB * half; p += kRopeThreads) {
-    const int t = small_div(p, half, rcp_half), band = p - t * half;
+  const float rcp_tw = 1.0f / (float)TW;
+  for (int p = tid; p < TB * TW; p += kRopeThreads) {
+    const int t = small_div(p, TW, rcp_tw), band = p - t * TW;
     float sn = 0.f, cs = 1.f;
     if (tok0 + t < ntok) {
       int b, l;
       batch_pos(t, b, l);
-      const int axis = a.n_axes > 1 ? band % a.n_axes : 0;
-      const float pos = (float)a.positions[((int64_t)axis * a.B + b) * a.L + l];
-      rope_sincos(__fdiv_rn(pos, a.timescale[band]), sn, cs);
-      if (a.inverse) sn = -sn;
+      if constexpr (TABLES) {
+        const int64_t at = ((int64_t)b * a.L + l) * a.D + band;
+        sn = (float)reinterpret_cast<const T *>(a.sin_t)[at];
+        cs = (float)reinterpret_cast<const T *>(a.cos_t)[at];
+      } else {
+        const int axis = a.n_axes > 1 ? band % a.n_axes : 0;
+        const float pos = (float)a.positions[((int64_t)axis * a.B + b) * a.L + l];
+        rope_sincos(__fdiv_rn(pos, a.timescale[band]), sn, cs);
+        if (a.inverse) sn = -sn;
+      }
     }
     sin_s[p] = sn;
     cos_s[p] = cs;
@@ -124,7 +135,7 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeArgs a, co
 #pragma clang fp contract(off)  // products and sums rounded one by one, as a framework's elementwise ops do
     const T *src[kRopeUnroll];
     T *dst[kRopeUnroll];
-    const T *wgt[kRopeUnroll];
+    const float *wgt[kRopeUnroll];
     int trig[kRopeUnroll];  // index of the item's first sine / cosine
     bool live[kRopeUnroll];
     Vec<T, V> x1[kRopeUnroll], x2[kRopeUnroll];
@@ -147,9 +158,9 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeArgs a, co
       src[u] = reinterpret_cast<const T *>(is_k ? a.k.ptr : a.q.ptr) + (is_k ? o.k : o.q) + h * sh_in + c * V;
       dst[u] = reinterpret_cast<T *>(const_cast<void *>(is_k ? a.k_out.ptr : a.q_out.ptr)) +
                (is_k ? o.k_out : o.q_out) + h * sh_out + c * V;
-      const void *w = is_k ? a.k_w : a.q_w;
-      wgt[u] = w ? reinterpret_cast<const T *>(w) + c * V : nullptr;
-      trig[u] = t * half + c * V;
+      const float *w = is_k ? a.k_w : a.q_w;
+      wgt[u] = w ? w + c * V : nullptr;
+      trig[u] = t * TW + c * V;
       if (live[u]) {
         x1[u] = *reinterpret_cast<const Vec<T, V> *>(src[u]);
         x2[u] = *reinterpret_cast<const Vec<T, V> *>(src[u] + half);
@@ -172,21 +183,45 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeArgs a, co
         for (int e = 0; e < V; ++e) ss += f1[e] * f1[e] + f2[e] * f2[e];
         for (int o = 1; o < lpr; o <<= 1) ss += __shfl_xor(ss, o, 64);
         const float r = 1.0f / sqrtf(ss / (float)a.D + a.eps);
-        const Vec<T, V> w1 = *reinterpret_cast<const Vec<T, V> *>(wgt[u]);
-        const Vec<T, V> w2 = *reinterpret_cast<const Vec<T, V> *>(wgt[u] + half);
+        const float *w1 = wgt[u], *w2 = wgt[u] + half;
+        if (a.norm_kind == BCATTN_NORM_GEMMA3) {
 #pragma unroll
-        for (int e = 0; e < V; ++e) {  // rounded to the element type, as the norm module returns it
-          f1[e] = (float)(T)((f1[e] * r) * (1.0f + (float)w1.v[e]));
-          f2[e] = (float)(T)((f2[e] * r) * (1.0f + (float)w2.v[e]));
+          for (int e = 0; e < V; ++e) {  // x * r * (1 + w), rounded to the element type as the module returns it
+            f1[e] = (float)(T)((f1[e] * r) * (1.0f + w1[e]));
+            f2[e] = (float)(T)((f2[e] * r) * (1.0f + w2[e]));
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < V; ++e) {  // w * (x * r rounded to the element type), rounded again
+            f1[e] = (float)(T)(w1[e] * (float)(T)(f1[e] * r));
+            f2[e] = (float)(T)(w2[e] * (float)(T)(f2[e] * r));
+          }
         }
       }
       const float *sp = sin_s + trig[u], *cp = cos_s + trig[u];
       Vec<T, V> y1, y2;
+      if constexpr (TABLES) {
+        // q * cos + rotate_half(q) * sin with rotate_half(q) = (-x2, x1), each step in the element
+        // type; its gradient is g * cos + (g2 * sin2, -g1 * sin1)
+        const float *sp2 = sp + half, *cp2 = cp + half;
+        auto rt = [](float x) __attribute__((always_inline)) { return (float)(T)x; };
 #pragma unroll
-      for (int e = 0; e < V; ++e) {
-        const float sn = sp[e], cs = cp[e];
-        y1.v[e] = (T)(f1[e] * cs - f2[e] * sn);
-        y2.v[e] = (T)(f2[e] * cs + f1[e] * sn);
+        for (int e = 0; e < V; ++e) {
+          if (!a.inverse) {
+            y1.v[e] = (T)(rt(f1[e] * cp[e]) + rt(-f2[e] * sp[e]));
+            y2.v[e] = (T)(rt(f2[e] * cp2[e]) + rt(f1[e] * sp2[e]));
+          } else {
+            y1.v[e] = (T)(rt(f1[e] * cp[e]) + rt(f2[e] * sp2[e]));
+            y2.v[e] = (T)(rt(f2[e] * cp2[e]) + rt(-f1[e] * sp[e]));
+          }
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          const float sn = sp[e], cs = cp[e];
+          y1.v[e] = (T)(f1[e] * cs - f2[e] * sn);
+          y2.v[e] = (T)(f2[e] * cs + f1[e] * sn);
+        }
       }
       *reinterpret_cast<Vec<T, V> *>(dst[u]) = y1;
       *reinterpret_cast<Vec<T, V> *>(dst[u] + half) = y2;
@@ -200,15 +235,22 @@ static void launch_rope_t(const RopeArgs &a, int rows, hipStream_t st) {
   const int TB = rope_tokens(a.D, rows * lpr);
   const int64_t ntok = (int64_t)a.B * a.L;
   const dim3 grid((unsigned)((ntok + TB - 1) / TB)), block(kRopeThreads);
-  const size_t lds = (size_t)TB * a.D * sizeof(float) + (size_t)TB * sizeof(RopeToken);
+  const bool tables = a.cos_t != nullptr;
+  const size_t lds = (size_t)TB * a.D * sizeof(float) * (tables ? 2 : 1) + (size_t)TB * sizeof(RopeToken);
   const float rr = 1.0f / (float)rows, rl = 1.0f / (float)lpr;
+#define BCATTN_ROPE_LAUNCH(LPR_)                                                                     \
+  if (tables)                                                                                        \
+    hipLaunchKernelGGL((rope_kernel<T, V, LPR_, true>), grid, block, lds, st, a, TB, rr, rl);        \
+  else                                                                                               \
+    hipLaunchKernelGGL((rope_kernel<T, V, LPR_, false>), grid, block, lds, st, a, TB, rr, rl)
   switch (lpr) {
-    case 4: hipLaunchKernelGGL((rope_kernel<T, V, 4>), grid, block, lds, st, a, TB, rr, rl); break;
-    case 8: hipLaunchKernelGGL((rope_kernel<T, V, 8>), grid, block, lds, st, a, TB, rr, rl); break;
-    case 16: hipLaunchKernelGGL((rope_kernel<T, V, 16>), grid, block, lds, st, a, TB, rr, rl); break;
-    case 32: hipLaunchKernelGGL((rope_kernel<T, V, 32>), grid, block, lds, st, a, TB, rr, rl); break;
-    default: hipLaunchKernelGGL((rope_kernel<T, V, 0>), grid, block, lds, st, a, TB, rr, rl); break;
+    case 4: BCATTN_ROPE_LAUNCH(4); break;
+    case 8: BCATTN_ROPE_LAUNCH(8); break;
+    case 16: BCATTN_ROPE_LAUNCH(16); break;
+    case 32: BCATTN_ROPE_LAUNCH(32); break;
+    default: BCATTN_ROPE_LAUNCH(0); break;
   }
+#undef BCATTN_ROPE_LAUNCH
 }
 
 int launch_rope(const RopeArgs &a, int dtype, hipStream_t st) {

@@ -17,7 +17,7 @@ from pathlib import Path
 
 CSRC = Path(__file__).resolve().parent.parent / "csrc"
 LIB_PATH = CSRC / "libbcattn.so"
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 # status codes of include/bcattn.h
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_LAUNCH = 0, -1, -2, -3, -4
@@ -121,6 +121,8 @@ class RopeParams(ctypes.Structure):
         ("k_out", Tensor4),
         ("positions", ctypes.c_void_p),
         ("timescale", ctypes.c_void_p),
+        ("cos", ctypes.c_void_p),
+        ("sin", ctypes.c_void_p),
         ("q_norm_weight", ctypes.c_void_p),
         ("k_norm_weight", ctypes.c_void_p),
         ("B", ctypes.c_int32),
@@ -131,6 +133,7 @@ class RopeParams(ctypes.Structure):
         ("n_axes", ctypes.c_int32),
         ("dtype", ctypes.c_int32),
         ("inverse", ctypes.c_int32),
+        ("norm_kind", ctypes.c_int32),
         ("norm_eps", ctypes.c_float),
     ]
 

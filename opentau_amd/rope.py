@@ -6,6 +6,10 @@ function serves pi0, pi06 and pi07).  ``apply_rope_qk`` is the form a layer want
 queries and keys in one launch, optionally behind Gemma-3's per-head RMS norm
 (``src/opentau/policies/pi06/gemma3_with_expert.py:851-861``), optionally written
 straight into other storage such as the rows of a preallocated key cache.
+``apply_rotary_pos_emb`` is the rotation of cosmos3's expert
+(``src/opentau/policies/cosmos3/qwen3vl_with_expert.py:217-224``): cos / sin tables from the
+backbone's rotary module, arithmetic in the tensors' own type, optionally behind the expert's
+per-head RMS norm (``:85-102``).
 There is no CPU path: without the library or a HIP device the calls raise.
 """
 
@@ -19,6 +23,7 @@ from .flash_attn_hip import _loader
 from .flash_attn_hip import _check, _DTYPES, _stream, _t4
 
 _timescales: dict[tuple, torch.Tensor] = {}
+_NORM_KINDS = {"gemma3": 0, "qwen3": 1}  # enum bcattn_norm_kind
 
 
 def rope_timescale(head_dim: int, max_wavelength: float, device: torch.device) -> torch.Tensor:
@@ -71,9 +76,17 @@ def rope_raw(
     q_norm_weight: torch.Tensor | None = None,
     k_norm_weight: torch.Tensor | None = None,
     norm_eps: float = 1e-6,
+    norm_kind: str = "gemma3",
     inverse: bool = False,
+    cos: torch.Tensor | None = None,
+    sin: torch.Tensor | None = None,
 ):
-    """One call of ``bcattn_rope``.  Returns ``(q_out, k_out)`` (``None`` where the input is ``None``)."""
+    """One call of ``bcattn_rope``.  Returns ``(q_out, k_out)`` (``None`` where the input is ``None``).
+
+    ``q`` / ``k`` are ``(B, L, H, D)`` views.  With ``cos`` / ``sin`` (``(B, L, D)``, cast to the tensors'
+    dtype) the rotation is ``x * cos + rotate_half(x) * sin`` in that dtype and ``positions`` is ignored.
+    ``norm_kind``: ``"gemma3"`` (``x * r * (1 + w)``) or ``"qwen3"`` (``w * (x * r)``).
+    """
     lib = _loader.require_library()
     x = q if q is not None else k
     if x is None:
@@ -87,7 +100,16 @@ def rope_raw(
     b, length, d = x.shape[0], x.shape[1], x.shape[3]
     if q is not None and k is not None and (k.shape[0], k.shape[1], k.shape[3], k.dtype) != (b, length, d, q.dtype):
         raise RuntimeError(f"q {tuple(q.shape)} and k {tuple(k.shape)} differ in batch, length, head_dim or dtype")
-    pos, n_axes = _positions(positions, b, length)
+    tables = cos is not None or sin is not None
+    if tables:
+        if cos is None or sin is None or tuple(cos.shape) != (b, length, d) or cos.shape != sin.shape:
+            raise RuntimeError(f"cos and sin must both be (B, L, D) = {(b, length, d)}")
+        cos, sin = (t.to(device=x.device, dtype=x.dtype).contiguous() for t in (cos, sin))
+        pos, n_axes = None, 1
+    else:
+        pos, n_axes = _positions(positions, b, length)
+    if norm_kind not in _NORM_KINDS:
+        raise RuntimeError(f"norm_kind must be one of {sorted(_NORM_KINDS)}")
     if q is not None and q_out is None:
         q_out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     if k is not None and k_out is None:
@@ -100,12 +122,16 @@ def rope_raw(
         if w is not None and t is not None:
             if w.shape != (d,):
                 raise RuntimeError(f"{what} must be ({d},), got {tuple(w.shape)}")
-            w = w.detach().to(device=t.device, dtype=t.dtype).contiguous()
+            w = w.detach().to(device=t.device, dtype=torch.float32).contiguous()
         weights.append(w if t is not None else None)
-    ts = rope_timescale(d, max_wavelength, x.device)
+    ts = None if tables else rope_timescale(d, max_wavelength, x.device)
     p = _loader.RopeParams()
     p.q, p.k, p.q_out, p.k_out = _t4(q), _t4(k), _t4(q_out if q is not None else None), _t4(k_out if k is not None else None)
-    p.positions, p.timescale = pos.data_ptr(), ts.data_ptr()
+    if tables:
+        p.cos, p.sin = cos.data_ptr(), sin.data_ptr()
+    else:
+        p.positions, p.timescale = pos.data_ptr(), ts.data_ptr()
+    p.norm_kind = _NORM_KINDS[norm_kind]
     p.q_norm_weight = weights[0].data_ptr() if weights[0] is not None else None
     p.k_norm_weight = weights[1].data_ptr() if weights[1] is not None else None
     p.B, p.L, p.D = b, length, d
@@ -161,6 +187,41 @@ _op_rope.register_autograd(_rope_backward, setup_context=_rope_setup)
 _op_rope_qk.register_autograd(_rope_qk_backward, setup_context=_rope_setup)
 
 
+@torch.library.custom_op("bcattn::rope_tables", mutates_args=())
+def _op_rope_tables(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                    inverse: bool) -> tuple[torch.Tensor, torch.Tensor]:
+    return _rope_tables_bhsd(q, k, cos, sin, inverse=inverse)
+
+
+@_op_rope_tables.register_fake
+def _(q, k, cos, sin, inverse):
+    return q.new_empty(q.shape), k.new_empty(k.shape)
+
+
+def _rope_tables_setup(ctx, inputs, output):
+    ctx.save_for_backward(inputs[2], inputs[3])
+    ctx.inverse = inputs[4]
+
+
+def _rope_tables_backward(ctx, grad_q, grad_k):
+    cos, sin = ctx.saved_tensors
+    dq, dk = _op_rope_tables(grad_q.contiguous(), grad_k.contiguous(), cos, sin, not ctx.inverse)
+    return dq, dk, None, None, None
+
+
+_op_rope_tables.register_autograd(_rope_tables_backward, setup_context=_rope_tables_setup)
+
+
+def _rope_tables_bhsd(q, k, cos, sin, *, inverse=False, q_norm_weight=None, k_norm_weight=None, norm_eps=1e-6):
+    """``q (B, H, S, D)``, ``k (B, Hkv, S, D)`` -> rotated tensors of the same shape (new storage)."""
+    qo = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    ko = torch.empty(k.shape, dtype=k.dtype, device=k.device)
+    rope_raw(q.transpose(1, 2), k.transpose(1, 2), None, q_out=qo.transpose(1, 2), k_out=ko.transpose(1, 2),
+             cos=cos, sin=sin, inverse=inverse, q_norm_weight=q_norm_weight, k_norm_weight=k_norm_weight,
+             norm_eps=norm_eps, norm_kind="qwen3")
+    return qo, ko
+
+
 def _needs_graph(*ts: torch.Tensor) -> bool:
     return torch.compiler.is_compiling() or (torch.is_grad_enabled() and any(t.requires_grad for t in ts))
 
@@ -204,3 +265,41 @@ def apply_rope_qk(
         return _op_rope_qk(q, k, positions, float(max_wavelength), False)
     return rope_raw(q, k, positions, max_wavelength, q_out=q_out, k_out=k_out, q_norm_weight=q_norm_weight,
                     k_norm_weight=k_norm_weight, norm_eps=norm_eps)
+
+
+def apply_rotary_pos_emb(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    cos: torch.Tensor,
+    sin: torch.Tensor,
+    unsqueeze_dim: int = 1,
+    *,
+    q_norm_weight: torch.Tensor | None = None,
+    k_norm_weight: torch.Tensor | None = None,
+    norm_eps: float = 1e-6,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """``q * cos + rotate_half(q) * sin`` (and the same for ``k``) in one launch.
+
+    Signature and numerics of the ``apply_rotary_pos_emb`` that cosmos3's expert imports from
+    ``transformers`` (``src/opentau/policies/cosmos3/qwen3vl_with_expert.py:70``, called ``:224``):
+    ``cos`` / ``sin`` are ``(B, S, D)`` in the tensors' dtype, ``q`` / ``k`` are ``(B, H, S, D)`` with
+    ``unsqueeze_dim=1`` (the expert's layout) or ``(B, S, H, D)`` with ``unsqueeze_dim=2``; every product
+    and sum is rounded to that dtype.  Differentiable in ``q`` and ``k``.  With norm weights the expert's
+    per-head RMS norm (``ExpertRMSNorm``, ``:85-102``) runs in front, i.e. ``:217-224`` in one call
+    (inference only).
+    """
+    if unsqueeze_dim not in (1, 2):
+        raise RuntimeError("unsqueeze_dim must be 1 (B, H, S, D) or 2 (B, S, H, D)")
+    if unsqueeze_dim == 2:
+        q, k = q.transpose(1, 2), k.transpose(1, 2)
+    norm = q_norm_weight is not None or k_norm_weight is not None
+    if _needs_graph(q, k):
+        if norm:
+            raise RuntimeError("apply_rotary_pos_emb is differentiable / traceable only without norm weights")
+        qo, ko = _op_rope_tables(q, k, cos, sin, False)
+    else:
+        qo, ko = _rope_tables_bhsd(q, k, cos, sin, q_norm_weight=q_norm_weight, k_norm_weight=k_norm_weight,
+                                   norm_eps=norm_eps)
+    if unsqueeze_dim == 2:
+        qo, ko = qo.transpose(1, 2), ko.transpose(1, 2)
+    return qo, ko

@@ -21,6 +21,16 @@ What pins them (``tests/test_oracle_rope.py``):
                        axes against the closed form (band d follows axis d % A).
 * ``gemma3_rms_norm``  float64 closed form; weight 0 on unit-RMS rows is the identity; a scaled row
                        gives the same result (scale invariance up to eps).
+* ``apply_rotary_pos_emb``  (restates the function of that name in ``transformers``'
+                       ``models/qwen3_vl/modeling_qwen3_vl.py``, which
+                       ``src/opentau/policies/cosmos3/qwen3vl_with_expert.py:70`` imports and ``:224`` calls)
+                       the library routine itself where ``transformers`` is importable, bit for bit in
+                       bf16 and fp32; in fp32 with cos / sin of the same angles it equals ``apply_rope``
+                       and the complex closed form; and a bf16 case built so that rounding each
+                       product separately gives another answer than rounding the sum once.
+* ``expert_rms_norm``  (``ExpertRMSNorm.forward``, ``cosmos3/qwen3vl_with_expert.py:85-102``) float64
+                       closed form; weight 1 on unit-RMS rows is the identity; the two roundings
+                       (normalised value, then the product with the weight) shown on a bf16 case.
 
 No function here is "parity unpinned".
 """
@@ -81,3 +91,33 @@ def rope_closed_form(x, positions, max_wavelength: float = 10_000):
                     z = complex(float(x[b, l, h, i]), float(x[b, l, h, i + half])) * turn
                     out[b, l, h, i], out[b, l, h, i + half] = z.real, z.imag
     return out
+
+
+def rotate_half(x: torch.Tensor) -> torch.Tensor:
+    half = x.shape[-1] // 2
+    return torch.cat([-x[..., half:], x[..., :half]], dim=-1)
+
+
+def apply_rotary_pos_emb(q, k, cos, sin, unsqueeze_dim: int = 1):
+    """``x * cos + rotate_half(x) * sin`` for q and k, in the tensors' own dtype (each elementwise op rounds);
+    ``cos`` / ``sin`` ``(B, S, D)`` are broadcast over the head axis at ``unsqueeze_dim``."""
+    c, s = cos.unsqueeze(unsqueeze_dim), sin.unsqueeze(unsqueeze_dim)
+    return q * c + rotate_half(q) * s, k * c + rotate_half(k) * s
+
+
+def expert_rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    """``weight * (x * rsqrt(mean(x^2) + eps)).to(x.dtype)``, the statistics in fp32
+    (``cosmos3/qwen3vl_with_expert.py:97-102``)."""
+    xf = x.to(torch.float32)
+    xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    return (weight * xf.to(x.dtype)).to(x.dtype)
+
+
+def rope_tables(positions: torch.Tensor, head_dim: int, max_wavelength: float = 10_000, dtype=torch.float32):
+    """``(cos, sin)`` ``(B, S, D)`` of plain positions ``(B, S)`` with both halves alike, the layout the
+    rotary module of a Hugging Face text model returns (``emb = cat(freqs, freqs)``)."""
+    half = head_dim // 2
+    timescale = max_wavelength ** ((2.0 / head_dim) * torch.arange(half, dtype=torch.float32, device=positions.device))
+    freqs = positions.to(torch.float32).unsqueeze(-1) / timescale
+    emb = torch.cat([freqs, freqs], dim=-1)
+    return emb.cos().to(dtype), emb.sin().to(dtype)

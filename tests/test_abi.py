@@ -148,6 +148,9 @@ def test_fake_impl_gives_shapes_without_running_kernels():
         rq, rk = torch.ops.bcattn.rope_qk(q, k[:, :50], pos, 10000.0, False)
         assert rq.shape == q.shape and rk.shape == (2, 50, 1, 256) and rk.dtype == torch.bfloat16
         assert torch.ops.bcattn.rope(q, pos, 10000.0, True).shape == q.shape
+        qh, cs = q.transpose(1, 2), torch.empty(2, 50, 256, dtype=torch.bfloat16)
+        tq, tk = torch.ops.bcattn.rope_tables(qh, qh[:, :1], cs, cs, False)
+        assert tq.shape == qh.shape and tk.shape == (2, 1, 50, 256)
 
 
 def test_workloads_are_seeded_and_shaped():

@@ -178,6 +178,71 @@ def test_rope_full_training_shape_keeps_pair_norms():
     assert torch.equal(qb, want[0]) and torch.equal(kb, want[1])
 
 
+# --------------------------------------------------------------------------- #
+# the cos / sin form of cosmos3's expert (transformers' apply_rotary_pos_emb)
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("b,h,hkv,s,d", [(2, 16, 8, 50, 128), (1, 4, 1, 131, 256), (3, 2, 2, 5, 64)])
+def test_rotary_tables_form_is_bit_exact(dtype, b, h, hkv, s, d):
+    """Every product and sum rounds to the element type on both sides, from the same tables: same bits."""
+    q, k = g(randn((b, h, s, d), dtype, 1)), g(randn((b, hkv, s, d), dtype, 2))
+    cos, sin = oracle.rope_tables(g(positions(b, s, 3)), d, 1_000_000, dtype)
+    want_q, want_k = oracle.apply_rotary_pos_emb(q, k, cos, sin)
+    got_q, got_k = hip_rope.apply_rotary_pos_emb(q, k, cos, sin)
+    assert got_q.shape == q.shape and torch.equal(got_q, want_q) and torch.equal(got_k, want_k)
+    # (B, S, H, D) operands
+    q2, k2 = q.transpose(1, 2).contiguous(), k.transpose(1, 2).contiguous()
+    got_q2, got_k2 = hip_rope.apply_rotary_pos_emb(q2, k2, cos, sin, unsqueeze_dim=2)
+    assert torch.equal(got_q2, want_q.transpose(1, 2)) and torch.equal(got_k2, want_k.transpose(1, 2))
+    # tables with unlike halves (nothing in the call assumes cat(freqs, freqs))
+    cos2, sin2 = g(randn((b, s, d), dtype, 4)), g(randn((b, s, d), dtype, 5))
+    want = oracle.apply_rotary_pos_emb(q, k, cos2, sin2)
+    got = hip_rope.apply_rotary_pos_emb(q, k, cos2, sin2)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_rotary_tables_form_gradients(dtype):
+    b, h, hkv, s, d = 2, 8, 2, 37, 128
+    cos, sin = oracle.rope_tables(g(positions(b, s, 3)), d, 10_000, dtype)
+    q0, k0 = g(randn((b, h, s, d), dtype, 1)), g(randn((b, hkv, s, d), dtype, 2))
+    gq, gk = g(randn((b, h, s, d), dtype, 3)), g(randn((b, hkv, s, d), dtype, 4))
+
+    def grads(fn):
+        q, k = q0.clone().requires_grad_(True), k0.clone().requires_grad_(True)
+        qo, ko = fn(q, k, cos, sin)
+        torch.autograd.backward([qo, ko], [gq, gk])
+        return qo.detach(), ko.detach(), q.grad, k.grad
+
+    want, got = grads(oracle.apply_rotary_pos_emb), grads(hip_rope.apply_rotary_pos_emb)
+    for name, a, e in zip(("q", "k", "dq", "dk"), got, want):
+        assert torch.equal(a, e), name
+    traced = grads(torch.compile(hip_rope.apply_rotary_pos_emb, backend="aot_eager", fullgraph=True))
+    for a, e in zip(traced, got):
+        assert torch.equal(a, e)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_expert_norm_then_rotary_tables(dtype):
+    """cosmos3's expert attention, lines 217-224 of its module: per-head RMS norm of q and k, head-major
+    layout, the backbone's cos / sin."""
+    b, h, hkv, s, d = 2, 16, 8, 50, 128
+    q_bshd, k_bshd = g(randn((b, s, h, d), dtype, 1) * 2.0), g(randn((b, s, hkv, d), dtype, 2) * 0.5)
+    wq, wk = g(1.0 + randn((d,), torch.float32, 3) * 0.2).to(dtype), g(1.0 + randn((d,), torch.float32, 4) * 0.2).to(dtype)
+    cos, sin = oracle.rope_tables(g(positions(b, s, 5)), d, 1_000_000, dtype)
+    want = oracle.apply_rotary_pos_emb(oracle.expert_rms_norm(q_bshd, wq).transpose(1, 2),
+                                       oracle.expert_rms_norm(k_bshd, wk).transpose(1, 2), cos, sin)
+    got = hip_rope.apply_rotary_pos_emb(q_bshd.transpose(1, 2), k_bshd.transpose(1, 2), cos, sin,
+                                        q_norm_weight=wq, k_norm_weight=wk, norm_eps=1e-6)
+    for a, e, name in zip(got, want, ("q", "k")):
+        assert a.shape == e.shape
+        if dtype == torch.float32:
+            assert rel_l2(a, e) <= 1e-5, name
+        else:  # a row sum that differs in its last bit can move the norm's rounding to bf16
+            assert_close_bf16(a.float(), e.float(), name)
+            assert rel_l2(a.float(), e.float()) <= 2e-3 and float((a != e).float().mean()) <= 2e-2, name
+
+
 def test_rope_argument_errors():
     x = g(randn((1, 4, 2, 64), torch.bfloat16, 1))
     pos = g(torch.zeros(1, 4, dtype=torch.long))

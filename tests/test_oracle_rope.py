@@ -84,3 +84,63 @@ def test_gemma3_rms_norm_closed_form_and_special_cases():
     assert torch.allclose(rope.gemma3_rms_norm(unit, torch.zeros(64)), unit, atol=1e-5)
     assert torch.allclose(rope.gemma3_rms_norm(8.0 * x, w), rope.gemma3_rms_norm(x, w), atol=1e-5)
     assert rope.gemma3_rms_norm(x.bfloat16(), w.bfloat16()).dtype == torch.bfloat16
+
+
+def test_rotary_tables_form_equals_apply_rope_in_fp32_and_the_closed_form():
+    x = randn((2, 6, 3, 32), torch.float32, 8)
+    k = randn((2, 6, 1, 32), torch.float32, 9)
+    p = torch.randint(0, 40, (2, 6), generator=torch.Generator().manual_seed(4))
+    cos, sin = rope.rope_tables(p, 32)
+    qo, ko = rope.apply_rotary_pos_emb(x, k, cos, sin, unsqueeze_dim=2)
+    assert rel_l2(qo, rope.apply_rope(x, p)) <= 1e-6 and rel_l2(ko, rope.apply_rope(k, p)) <= 1e-6
+    assert rel_l2(qo, rope.rope_closed_form(x, p)) <= 1e-6
+    # head-major layout, unsqueeze_dim = 1
+    qh, kh = rope.apply_rotary_pos_emb(x.transpose(1, 2), k.transpose(1, 2), cos, sin)
+    assert torch.equal(qh.transpose(1, 2), qo) and torch.equal(kh.transpose(1, 2), ko)
+
+
+def test_rotary_tables_form_against_the_library_routine():
+    m = __import__("pytest").importorskip("transformers.models.qwen3_vl.modeling_qwen3_vl")
+    for dtype in (torch.bfloat16, torch.float32):
+        q, k = randn((2, 4, 7, 64), dtype, 10), randn((2, 2, 7, 64), dtype, 11)
+        p = torch.randint(0, 900, (2, 7), generator=torch.Generator().manual_seed(5))
+        cos, sin = rope.rope_tables(p, 64, 1_000_000, dtype)
+        want = m.apply_rotary_pos_emb(q, k, cos, sin)
+        got = rope.apply_rotary_pos_emb(q, k, cos, sin)
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+
+
+def test_rotary_tables_form_rounds_every_step_in_bf16():
+    bf = torch.bfloat16
+    x = torch.tensor([257.0, 3.0]).to(bf).reshape(1, 1, 1, 2)       # 257 -> 256 in bf16 (8 significant bits)
+    cos = torch.tensor([[[1.5, 1.5]]]).to(bf)
+    sin = torch.tensor([[[0.75, 0.75]]]).to(bf)
+    out, _ = rope.apply_rotary_pos_emb(x, x, cos, sin, unsqueeze_dim=2)
+    # first element: bf16(256 * 1.5) + bf16(-3 * 0.75) = 384 + (-2.25) = 381.75 -> bf16 382
+    # second: bf16(3 * 1.5) + bf16(256 * 0.75) = 4.5 + 192 = 196.5 -> bf16 196 (tie to even) ... exact sums
+    assert out.flatten().tolist() == [382.0, 196.0]
+    # a case where the separately rounded product matters: 1.0078125 * 1.0078125 = 1.01568... -> bf16 1.015625;
+    # 0.00390625 added after gives 1.01953125, a tie that goes to the even 1.015625, whereas the exact sum
+    # 1.01959... rounded once goes up to 1.0234375
+    x = torch.tensor([1.0078125, 0.00390625]).to(bf).reshape(1, 1, 1, 2)
+    cos = torch.tensor([[[1.0078125, 1.0]]]).to(bf)
+    sin = torch.tensor([[[-1.0, 0.0]]]).to(bf)
+    out, _ = rope.apply_rotary_pos_emb(x, x, cos, sin, unsqueeze_dim=2)
+    once = torch.tensor(1.0078125 * 1.0078125 + 0.00390625).to(bf)
+    assert float(out[0, 0, 0, 0]) == 1.015625 and float(once) == 1.0234375
+
+
+def test_expert_rms_norm_closed_form_and_roundings():
+    x = randn((2, 3, 4, 64), torch.float32, 12)
+    w = 1.0 + randn((64,), torch.float32, 13) * 0.1
+    xd = x.double()
+    want = w.double() * (xd / torch.sqrt((xd * xd).mean(-1, keepdim=True) + 1e-6))
+    assert rel_l2(rope.expert_rms_norm(x, w), want) <= 1e-6
+    unit = x / x.pow(2).mean(-1, keepdim=True).sqrt()
+    assert torch.allclose(rope.expert_rms_norm(unit, torch.ones(64)), unit, atol=1e-5)
+    # bf16: the normalised value is rounded before it meets the weight
+    xb, wb = x.bfloat16(), w.bfloat16()
+    xf = xb.float()
+    normed = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16()
+    assert torch.equal(rope.expert_rms_norm(xb, wb), (wb.float() * normed.float()).bfloat16())
+    assert rope.expert_rms_norm(xb, w).dtype == torch.bfloat16  # fp32 weight on a bf16 input
