@@ -228,25 +228,33 @@ def bench_rope(torch, dev, calls=50, warmup=5):
     from opentau_amd import rope
 
     out = {}
-    for name, (b, length, h, hkv, d) in {"c3": (32, 754, 8, 1, 256), "c5": (4, 4402, 64, 8, 128)}.items():
+    shapes = {"c3": (32, 754, 8, 1, 256, False), "c5": (4, 4402, 64, 8, 128, False),
+              "c5_cos_sin": (4, 4402, 64, 8, 128, True)}
+    for name, (b, length, h, hkv, d, tables) in shapes.items():
         gen = torch.Generator(device="cpu").manual_seed(0)
         q = torch.randn(b, length, h, d, generator=gen).to(dev, torch.bfloat16)
         k = torch.randn(b, length, hkv, d, generator=gen).to(dev, torch.bfloat16)
         pos = torch.arange(length, dtype=torch.int32, device=dev)[None].expand(b, length).contiguous()
+        kw = {}
+        if tables:  # cosmos3's form: cos / sin tables from the backbone, arithmetic in bf16
+            ang = pos[..., None].float() / (1e6 ** (torch.arange(d // 2, device=dev).float() * (2.0 / d)))
+            emb = torch.cat([ang, ang], -1)
+            kw = {"cos": emb.cos().to(torch.bfloat16), "sin": emb.sin().to(torch.bfloat16)}
         for _ in range(warmup):
-            rope.rope_raw(q, k, pos, q_out=q, k_out=k)
+            rope.rope_raw(q, k, pos, q_out=q, k_out=k, **kw)
         t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         t0.record()
         for _ in range(calls):
-            rope.rope_raw(q, k, pos, q_out=q, k_out=k)
+            rope.rope_raw(q, k, pos, q_out=q, k_out=k, **kw)
         t1.record()
         torch.cuda.synchronize()
         us = t0.elapsed_time(t1) * 1e3 / calls
-        nbytes = 2 * 2 * (q.numel() + k.numel()) + 4 * pos.numel()
+        nbytes = 2 * 2 * (q.numel() + k.numel()) + (2 * 2 * b * length * d if tables else 4 * pos.numel())
         gbps = nbytes / (us * 1e-6) / 1e9
         out[name] = {
-            "workload": f"rope of q and k in place, bf16 B{b} L{length} H{h} Hkv{hkv} D{d}",
+            "workload": f"rope of q and k in place{' from cos/sin tables' if tables else ''}, "
+                        f"bf16 B{b} L{length} H{h} Hkv{hkv} D{d}",
             "us_per_call": round(us, 2),
             "algorithmic_bytes": nbytes,
             "gbps": round(gbps, 1),
