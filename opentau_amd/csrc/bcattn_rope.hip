@@ -198,12 +198,25 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeArgs a, co
           }
         }
       }
-      const float *sp = sin_s + trig[u], *cp = cos_s + trig[u];
+      // V consecutive floats of LDS, 16-byte aligned (V, D/2 and the per-token widths are multiples of 4)
+      auto lds_floats = [](const float *p, float(&o)[V]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int x = 0; x < V / 4; ++x) {
+          const f32x4 t = *reinterpret_cast<const f32x4 *>(p + 4 * x);
+#pragma unroll
+          for (int y = 0; y < 4; ++y) o[4 * x + y] = t[y];
+        }
+      };
+      float sp[V], cp[V];
+      lds_floats(sin_s + trig[u], sp);
+      lds_floats(cos_s + trig[u], cp);
       Vec<T, V> y1, y2;
       if constexpr (TABLES) {
         // q * cos + rotate_half(q) * sin with rotate_half(q) = (-x2, x1), each step in the element
         // type; its gradient is g * cos + (g2 * sin2, -g1 * sin1)
-        const float *sp2 = sp + half, *cp2 = cp + half;
+        float sp2[V], cp2[V];
+        lds_floats(sin_s + trig[u] + half, sp2);
+        lds_floats(cos_s + trig[u] + half, cp2);
         auto rt = [](float x) __attribute__((always_inline)) { return (float)(T)x; };
 #pragma unroll
         for (int e = 0; e < V; ++e) {
