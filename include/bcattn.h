@@ -172,6 +172,26 @@ int bcattn_fwd(const bcattn_fwd_params *p, void *stream);
  */
 int bcattn_fwd_kvcache(const bcattn_fwd_params *p, void *stream);
 
+/*
+ * The same call as bcattn_fwd_kvcache for callers that cannot allocate device memory
+ * at all (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): it has no counterpart in the reference.  The workspace (tile summaries,
+ * merged ids, split-key partials) is a fixed array of BCATTN_STATIC_SCRATCH_BYTES bytes
+ * of device memory inside the library, one copy per GPU, held until the process ends;
+ * p->workspace and p->workspace_bytes are not read.  The caller still passes q, k, v,
+ * k1, v1, o (and lse).  A call whose bcattn_fwd_kvcache_workspace_bytes() exceeds the
+ * array returns BCATTN_ERR_WORKSPACE with a message; fp32 is not covered
+ * (BCATTN_ERR_UNSUPPORTED).  No hipMalloc / hipFree or other allocating routine is
+ * called.  All calls on one GPU share that GPU's array: two calls that overlap in time
+ * on one GPU (different streams or threads) race, and summary_ready != 0 means "the
+ * array still holds the summary of the previous call on this GPU, whose masks and
+ * shape were the same".  The first call on a device looks up the array's address
+ * (hipGetSymbolAddress) and raises the kernels' dynamic-LDS limit; make that call
+ * outside graph capture.
+ */
+#define BCATTN_STATIC_SCRATCH_BYTES (32u << 20)
+int bcattn_fwd_kvcache_static(const bcattn_fwd_params *p, void *stream);
+
 /* Replaces flash_bwd (flash_blockmask.cu:1210-1327). */
 int bcattn_bwd(const bcattn_bwd_params *p, void *stream);
 

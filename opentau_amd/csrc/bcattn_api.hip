@@ -192,6 +192,31 @@ static int fwd_prepare(const bcattn_fwd_params *p, FwdArgs &a, char *&ws, hipStr
   return BCATTN_OK;
 }
 
+// ---- scratch of the allocation-free entry point ------------------------------------
+// Device memory that exists from the moment the code object is loaded on a GPU until the
+// process ends; every GPU holds its own copy at its own address.  In host code the array's
+// name is only a handle for hipGetSymbolAddress: the address that kernels and copies take
+// is the one that call returns, looked up once per device (with that device current).
+static __device__ __align__(256) unsigned char scratch[BCATTN_STATIC_SCRATCH_BYTES];
+
+static void *static_scratch() {
+  static std::atomic<void *> per_device[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    fail(BCATTN_ERR_LAUNCH, "no current HIP device (or device index above 63)");
+    return nullptr;
+  }
+  void *ptr = per_device[dev].load(std::memory_order_acquire);
+  if (ptr != nullptr) return ptr;
+  const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || ptr == nullptr) {
+    fail(BCATTN_ERR_LAUNCH, "hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+    return nullptr;
+  }
+  per_device[dev].store(ptr, std::memory_order_release);
+  return ptr;
+}
+
 }  // namespace bcattn
 
 using namespace bcattn;
@@ -242,18 +267,17 @@ int bcattn_fwd(const bcattn_fwd_params *p, void *stream) {
   return BCATTN_OK;
 }
 
-int bcattn_fwd_kvcache(const bcattn_fwd_params *p, void *stream) {
-  int rc = check_fwd(p);
-  if (rc) return rc;
-  if (p->B == 0) return BCATTN_OK;
-  if (!is16(p->dtype)) return bcattn_fwd(p, stream);
+// The KV-cached forward over a workspace of `ws_bytes` bytes at `ws_ptr` (the caller's, or the
+// library's static scratch).
+static int fwd_kvcache_over(const bcattn_fwd_params *p, void *ws_ptr, size_t ws_bytes, void *stream) {
+  int rc;
   const size_t need = bcattn_fwd_kvcache_workspace_bytes(p);
-  if (p->workspace == nullptr || p->workspace_bytes < need || !aligned16(p->workspace))
+  if (ws_ptr == nullptr || ws_bytes < need || !aligned16(ws_ptr))
     return fail(BCATTN_ERR_WORKSPACE, "kvcache forward needs %zu bytes of 16-byte aligned workspace, got %zu",
-                need, p->workspace ? p->workspace_bytes : (size_t)0);
+                need, ws_ptr ? ws_bytes : (size_t)0);
   hipStream_t st = reinterpret_cast<hipStream_t>(stream);
   FwdArgs a = fwd_args(p);
-  char *ws = reinterpret_cast<char *>(p->workspace);
+  char *ws = reinterpret_cast<char *>(ws_ptr);
   if ((rc = fwd_prepare(p, a, ws, st))) return rc;
   SplitArgs s;
   s.tiles_per_split = 0;
@@ -266,6 +290,31 @@ int bcattn_fwd_kvcache(const bcattn_fwd_params *p, void *stream) {
                               : bf16::launch_fwd_kvcache_mfma(a, s, p->D, st);
   if (rc) return fail(rc, "kvcache forward launch failed (D=%d)", p->D);
   return BCATTN_OK;
+}
+
+int bcattn_fwd_kvcache(const bcattn_fwd_params *p, void *stream) {
+  int rc = check_fwd(p);
+  if (rc) return rc;
+  if (p->B == 0) return BCATTN_OK;
+  if (!is16(p->dtype)) return bcattn_fwd(p, stream);
+  return fwd_kvcache_over(p, p->workspace, p->workspace_bytes, stream);
+}
+
+int bcattn_fwd_kvcache_static(const bcattn_fwd_params *p, void *stream) {
+  int rc = check_fwd(p);
+  if (rc) return rc;
+  if (p->B == 0) return BCATTN_OK;
+  if (!is16(p->dtype))
+    return fail(BCATTN_ERR_UNSUPPORTED, "the allocation-free call covers bf16 and fp16 only (dtype %d)", p->dtype);
+  const size_t need = bcattn_fwd_kvcache_workspace_bytes(p);
+  if (need > (size_t)BCATTN_STATIC_SCRATCH_BYTES)
+    return fail(BCATTN_ERR_WORKSPACE,
+                "this call needs %zu bytes of scratch; the library's static scratch holds %zu "
+                "(use bcattn_fwd_kvcache with a workspace of the caller's)",
+                need, (size_t)BCATTN_STATIC_SCRATCH_BYTES);
+  void *ws = static_scratch();
+  if (ws == nullptr) return BCATTN_ERR_LAUNCH;  // (message set by static_scratch)
+  return fwd_kvcache_over(p, ws, (size_t)BCATTN_STATIC_SCRATCH_BYTES, stream);
 }
 
 int bcattn_bwd(const bcattn_bwd_params *p, void *stream) {

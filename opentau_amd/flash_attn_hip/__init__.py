@@ -181,6 +181,7 @@ def forward_raw(
     summary_ready: bool = False,
     out: torch.Tensor | None = None,
     want_lse: bool = True,
+    static_scratch: bool = False,
 ):
     """One forward through the C ABI.  Returns ``(out (B,Sq,H,D), lse (B,H,Sq) | None)``.
 
@@ -189,11 +190,16 @@ def forward_raw(
     an earlier call with the same mask (``summary_ready=True``).  When segment 0
     has fewer batch entries than ``q`` (``B = n * k.shape[0]``), batch entry ``b``
     reads entry ``b // n`` of it: the un-expanded prefix cache of best-of-N
-    sampling (``src/opentau/policies/candidates.py:114-127``).
+    sampling (``src/opentau/policies/candidates.py:114-127``).  ``static_scratch`` (with
+    ``kvcache``) takes ``bcattn_fwd_kvcache_static``: the library's own fixed scratch instead of
+    a workspace, so that the call itself allocates nothing when ``out`` is given and
+    ``want_lse`` is off.
     """
     lib = _loader.require_library()
     _check_inputs(q, k, v)
     extra = _head_dim_padding(q)
+    if static_scratch and (extra or not kvcache or workspace is not None):
+        raise RuntimeError("static_scratch goes with kvcache=True, no workspace and a head_dim the kernels take")
     if extra:
         o, lse = forward_raw(_padded(q, extra), _padded(k, extra), _padded(v, extra), q_blk, k_blk, q_valid, k_valid,
                              scale, _padded(k_new, extra), _padded(v_new, extra), kvcache=kvcache,
@@ -227,6 +233,10 @@ def forward_raw(
     p.dtype, p.scale = code, float(scale)
     p.summary_ready = 1 if summary_ready else 0
     p.kv_share = share
+    if static_scratch:
+        with torch.cuda.device(q.device):
+            _check(lib.bcattn_fwd_kvcache_static(ctypes.byref(p), _stream(q.device)), lib)
+        return out, lse
     size_fn = lib.bcattn_fwd_kvcache_workspace_bytes if kvcache else lib.bcattn_fwd_workspace_bytes
     need = size_fn(ctypes.byref(p))
     if workspace is None or workspace.numel() < need:

@@ -23,6 +23,7 @@ ABI_VERSION = 3
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_LAUNCH = 0, -1, -2, -3, -4
 DTYPE_F32, DTYPE_BF16, DTYPE_F16 = 0, 1, 2
 BWD_DELTA, BWD_DQ, BWD_DKV = 1, 2, 4
+STATIC_SCRATCH_BYTES = 32 << 20  # BCATTN_STATIC_SCRATCH_BYTES
 
 EXPORTS = (
     "bcattn_abi_version",
@@ -32,6 +33,7 @@ EXPORTS = (
     "bcattn_bwd_workspace_bytes",
     "bcattn_fwd",
     "bcattn_fwd_kvcache",
+    "bcattn_fwd_kvcache_static",
     "bcattn_bwd",
     "bcattn_rope",
 )
@@ -157,7 +159,8 @@ def _bind(lib: ctypes.CDLL) -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = ctypes.c_size_t
         fn.argtypes = [ctypes.POINTER(st)]
-    for name, st in (("bcattn_fwd", FwdParams), ("bcattn_fwd_kvcache", FwdParams), ("bcattn_bwd", BwdParams),
+    for name, st in (("bcattn_fwd", FwdParams), ("bcattn_fwd_kvcache", FwdParams),
+                     ("bcattn_fwd_kvcache_static", FwdParams), ("bcattn_bwd", BwdParams),
                      ("bcattn_rope", RopeParams)):
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int

@@ -1,0 +1,95 @@
+"""The allocation-free KV-cached forward (``bcattn_fwd_kvcache_static``) against the entry point it
+is a variant of (``bcattn_fwd_kvcache`` with a caller-owned workspace), through the C ABI.
+
+Both run the same kernels over the same workspace layout, so the outputs must be bit-identical
+(stricter than the acceptance bar of rel-L2 <= 1e-2, max-abs <= 2e-2 for bf16).  Two calls in a row,
+the second with a smaller input: the library's scratch keeps the first call's contents, and the
+second call must not read any of it.  Collected last on purpose.
+"""
+
+import ctypes
+
+import pytest
+import torch
+
+from opentau_amd import flash_attn_hip as fa
+from opentau_amd.flash_attn_hip import _loader
+from oracle import eager
+
+from helpers import assert_close_bf16, randn
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_kernels():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    if not fa.is_available():
+        raise RuntimeError(f"HIP kernels unavailable on a GPU box: {fa.load_error()}")
+
+
+def _case(b, sq, h, hkv, d, cross, dtype, seed):
+    dev = torch.device("cuda:0")
+    q = randn((b, sq, h, d), dtype, seed)
+    kc, vc = randn((b, cross, hkv, d), dtype, seed + 1), randn((b, cross, hkv, d), dtype, seed + 2)
+    kn, vn = randn((b, sq, hkv, d), dtype, seed + 3), randn((b, sq, hkv, d), dtype, seed + 4)
+    pad = torch.ones(b, sq, dtype=torch.bool)
+    att = torch.zeros(b, sq, dtype=torch.int32)
+    att[:, 0] = 1
+    cross_pad = torch.ones(b, cross, dtype=torch.bool)
+    gen = torch.Generator().manual_seed(seed)
+    for i in range(b):  # right-padded cached text, a different length per sample
+        cross_pad[i, cross - int(torch.randint(0, cross // 3, (1,), generator=gen)):] = False
+    ids = fa.make_att_block_ids(pad, att, cross, cross_pad)
+    cpu = (q, kc, vc, kn, vn, ids)
+    gpu = tuple(t.to(dev) for t in (q, kc, vc, kn, vn)) + (tuple(t.to(dev) for t in ids),)
+    return cpu, gpu
+
+
+def _both(gpu, scale):
+    q, kc, vc, kn, vn, ids = gpu
+    want, lse_w = fa.forward_raw(q, kc, vc, *ids, scale, kn, vn, kvcache=True)
+    out = torch.full_like(q, float("nan"))
+    got, lse_g = fa.forward_raw(q, kc, vc, *ids, scale, kn, vn, kvcache=True, static_scratch=True, out=out)
+    torch.cuda.synchronize()
+    return want, lse_w, got, lse_g
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_static_scratch_call_matches_the_workspace_call_twice_in_a_row(dtype):
+    # first the pi0.5 denoise shape, then a smaller one (fewer samples, shorter cache, other head_dim)
+    shapes = [(8, 50, 8, 1, 256, 968), (2, 33, 8, 2, 128, 200)]
+    for n, (b, sq, h, hkv, d, cross) in enumerate(shapes):
+        cpu, gpu = _case(b, sq, h, hkv, d, cross, dtype, seed=100 + n)
+        scale = d**-0.5
+        want, lse_w, got, lse_g = _both(gpu, scale)
+        assert torch.equal(got, want), f"call {n}: outputs differ from the workspace call"
+        assert torch.equal(lse_g, lse_w), f"call {n}: LSE differs from the workspace call"
+        # and both against the oracle on the concatenated keys, at the acceptance bar
+        q, kc, vc, kn, vn, ids = cpu
+        ref = eager.eager_from_block_ids(q, torch.cat([kc, kn], 1), torch.cat([vc, vn], 1), *ids, scale)
+        assert_close_bf16(got.float().cpu(), ref.float().reshape(got.shape), f"call {n} vs oracle")
+
+
+def test_static_scratch_refuses_what_does_not_fit_and_reuses_its_summary():
+    lib = _loader.require_library()
+    dev = torch.device("cuda:0")
+    # more scratch than the array holds (255 row tiles, each split in two): a clear error, nothing launched
+    b, sq, h, hkv, d, cross = 255, 50, 1, 1, 256, 128
+    q = torch.zeros(b, sq, h, d, dtype=torch.bfloat16, device=dev)
+    kc = torch.zeros(b, cross, hkv, d, dtype=torch.bfloat16, device=dev)
+    kn = torch.zeros(b, sq, hkv, d, dtype=torch.bfloat16, device=dev)
+    ids = [t.to(dev) for t in fa.make_att_block_ids(torch.ones(b, sq, dtype=torch.bool), torch.zeros(b, sq),
+                                                    cross, torch.ones(b, cross, dtype=torch.bool))]
+    assert fa.kvcache_workspace_bytes(b, sq, cross, sq, h, hkv, d) > _loader.STATIC_SCRATCH_BYTES
+    with pytest.raises(RuntimeError, match="static scratch holds"):
+        fa.forward_raw(q, kc, kc, *ids, 0.0625, kn, kn, kvcache=True, static_scratch=True)
+    assert b"scratch" in lib.bcattn_last_error()
+    # summary_ready: the array still holds the previous call's summary (same mask): same bits
+    cpu, gpu = _case(4, 50, 8, 1, 256, 968, torch.bfloat16, seed=7)
+    q, kc, vc, kn, vn, ids = gpu
+    first, _ = fa.forward_raw(q, kc, vc, *ids, 0.0625, kn, vn, kvcache=True, static_scratch=True)
+    again, _ = fa.forward_raw(q, kc, vc, *ids, 0.0625, kn, vn, kvcache=True, static_scratch=True, summary_ready=True)
+    torch.cuda.synchronize()
+    assert torch.equal(first, again)
