@@ -10,13 +10,12 @@
  * over raw device pointers, element strides and an explicit HIP stream.  No
  * torch types, no device allocation: the caller owns every buffer (outputs and
  * the workspace), no pointer is retained after return, and every call is
- * asynchronous with respect to the host on the stream it is given.  The one
- * thing the library keeps is a helper stream and two events per device (and
- * 16-bit element type), made on the first bcattn_bwd call that computes all gradients: its two large
- * kernels run side by side, forked from and joined to the given stream, so
- * work enqueued on that stream afterwards still sees all of the call's results
- * (BCATTN_SERIAL_BACKWARD=1 in the environment keeps everything on the given
- * stream).
+ * asynchronous with respect to the host on the stream it is given, and uses no
+ * other stream.  The library keeps no state between calls besides the thread-local
+ * error text (and, per device, the fixed scratch of bcattn_fwd_kvcache_static).
+ * A bcattn_bwd call that computes all gradients runs dQ and dK/dV as one launch
+ * (BCATTN_SERIAL_BACKWARD=1 in the environment launches its kernels one by one,
+ * which is how a profiler sees each alone).
  *
  * Mask rule (flash_attn_cuda/__init__.py:27-28):
  *     attend(i,j) = q_valid[i] && k_valid[j] && k_blk[j] <= q_blk[i]

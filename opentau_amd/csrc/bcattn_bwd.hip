@@ -13,7 +13,7 @@
 //           at 256 as two launches, dV then dK), or, at head_dim 128 and long rows,
 //           two waves per 32 keys split them and pass P through LDS
 // P is recomputed from the saved log-sum-exp: P = exp2(scale*log2e*S - log2e*LSE).
-// A call that computes dQ and dK/dV runs the two kernels side by side on two streams.
+// A call that computes dQ and dK/dV runs both in one launch, the dK/dV workgroups first.
 //
 // As in the forward, the 32x32 accumulator of the first product is already the B
 // operand of the second, so P / dS never leave registers inside a wave.  Streamed tiles
@@ -22,7 +22,6 @@
 // sequence axis (K^T, Q^T, dO^T) is read from the same row-major tile with the
 // transposing LDS read.
 #include <cstdlib>
-#include <mutex>
 
 #include "bcattn_tiles.h"
 
@@ -72,8 +71,9 @@ struct BwdStages {
 };
 
 // ---- dQ ------------------------------------------------------------------------
+// `block`: the workgroup's index among the dQ workgroups (the launch may hold other work in front)
 template <int D, int NW>
-__global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
+__device__ __forceinline__ void bwd_dq_body(const BwdArgs &a, const unsigned block) {
   using T = Tile<D>;
   constexpr int NT = 64 * NW, BM = 32 * NW;
   constexpr int DK = D / 16, DB = D / 32;
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   const int R = a.G * a.Sq;
   const int ntile_r = (R + BM - 1) / BM;
   const int nitems = ntile_r * a.Hkv * a.B;
-  int bid = xcd_item(blockIdx.x, nitems);
+  int bid = xcd_item(block, nitems);
   if (bid >= nitems) return;
   const int tile = __builtin_amdgcn_readfirstlane(bid % ntile_r);
   bid /= ntile_r;
@@ -271,6 +271,12 @@ __global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
   store_rows_whole_lines<D>(dq, a.scale, rowok ? optr : nullptr, smem + wave * kOutBytes<D>, lane);
 }
 
+template <int D, int NW>
+__global__ __launch_bounds__(64 * NW) void bwd_dq_kernel(const BwdArgs a) {
+  warm_kernel_arguments<sizeof(BwdArgs)>();
+  bwd_dq_body<D, NW>(a, blockIdx.x);
+}
+
 template <int D>
 constexpr size_t dq_smem_bytes() {
   return StageLayout<D, BwdStages<D>::value, 256>::kBytes;
@@ -284,7 +290,7 @@ constexpr size_t dq_smem_bytes() {
 constexpr int kModeBoth = 0, kModeDV = 1, kModeDK = 2;
 
 template <int D, int NW, int MODE>
-__global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
+__device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, const unsigned block) {
   using T = Tile<D>;
   constexpr bool WANT_DV = MODE != kModeDK, WANT_DK = MODE != kModeDV;
   constexpr int NT = 64 * NW, BK = 32 * NW;
@@ -302,7 +308,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   const int Sk = a.Sk, Sq = a.Sq, Sqp = a.Sq_pad;
   const int nkt = (Sk + BK - 1) / BK;
   const int nitems = nkt * a.Hkv * a.B;
-  int bid = xcd_item(blockIdx.x, nitems);
+  int bid = xcd_item(block, nitems);
   if (bid >= nitems) return;
   const int kt = __builtin_amdgcn_readfirstlane(bid % nkt);
   bid /= nkt;
@@ -576,6 +582,12 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   }
 }
 
+template <int D, int NW, int MODE>
+__global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
+  warm_kernel_arguments<sizeof(BwdArgs)>();
+  bwd_dkv_body<D, NW, MODE>(a, blockIdx.x);
+}
+
 // ---- dK / dV with paired waves --------------------------------------------------------
 // Two waves share 32 keys and split the work of a 32-query half tile in two equal parts:
 //   the P wave   holds the K fragments and the dV accumulators:
@@ -596,7 +608,7 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
 // tile k+1 before B(2k+1); tile k+2 is requested after B(2k), when tile k-1, whose
 // stage it takes, was last used before B(2k).
 template <int D, int NP>
-__global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a) {
+__device__ __forceinline__ void bwd_dkv_pair_body(const BwdArgs &a, const unsigned block) {
   using T = Tile<D>;
   constexpr int NW = 2 * NP, NT = 64 * NW, BK = 32 * NP;
   constexpr int DK = D / 16, DB = D / 32;
@@ -616,7 +628,7 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
   const int Sk = a.Sk, Sq = a.Sq, Sqp = a.Sq_pad;
   const int nkt = (Sk + BK - 1) / BK;
   const int nitems = nkt * a.Hkv * a.B;
-  int bid = xcd_item(blockIdx.x, nitems);
+  int bid = xcd_item(block, nitems);
   if (bid >= nitems) return;
   const int kt = __builtin_amdgcn_readfirstlane(bid % nkt);
   bid /= nkt;
@@ -1036,6 +1048,51 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
 }
 
 template <int D, int NP>
+__global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a) {
+  warm_kernel_arguments<sizeof(BwdArgs)>();
+  bwd_dkv_pair_body<D, NP>(a, blockIdx.x);
+}
+
+// dK/dV and dQ in one launch.  The two are independent, and each alone leaves part of the chip idle
+// while its last workgroups finish (a workgroup holds most of a CU's LDS, so a grid is a small number
+// of "rounds" of one workgroup per CU, and a dK/dV workgroup runs several times as long as a dQ
+// workgroup).  Workgroups are handed out in index order: the dK/dV workgroups take the first
+// indices, so all of the long ones start first and the short dQ workgroups fill the CUs as they
+// come free, up to the very end.  (Every role's share of the grid is a multiple of 8 workgroups, so
+// each keeps its own XCD mapping.)
+template <int D, int NWQ, int NP>
+__global__ __launch_bounds__(128 * NP) void bwd_dkv_dq_kernel(const BwdArgs a, const unsigned ndkv) {
+  static_assert(64 * NWQ == 128 * NP, "both roles use the same workgroup size");
+  warm_kernel_arguments<sizeof(BwdArgs) + sizeof(unsigned)>();
+  if (blockIdx.x < ndkv)
+    bwd_dkv_pair_body<D, NP>(a, blockIdx.x);
+  else
+    bwd_dq_body<D, NWQ>(a, blockIdx.x - ndkv);
+}
+
+// The same for the single-wave dK/dV forms.  TWO: dK/dV as two sets of `ndkv` workgroups (dV alone,
+// then dK alone: the form head_dim 256 takes).  (Measured on the pi0.5 / pi0.6 training shapes: with
+// the dK set in front of the dV set the step is 7 % slower; dQ workgroups placed between the two sets
+// change nothing.)
+template <int D, int NW, bool TWO>
+__global__ __launch_bounds__(64 * NW) void bwd_dkv1_dq_kernel(const BwdArgs a, const unsigned ndkv) {
+  warm_kernel_arguments<sizeof(BwdArgs) + sizeof(unsigned)>();
+  if constexpr (TWO) {
+    if (blockIdx.x < ndkv)
+      bwd_dkv_body<D, NW, kModeDV>(a, blockIdx.x);
+    else if (blockIdx.x < 2 * ndkv)
+      bwd_dkv_body<D, NW, kModeDK>(a, blockIdx.x - ndkv);
+    else
+      bwd_dq_body<D, NW>(a, blockIdx.x - 2 * ndkv);
+  } else {
+    if (blockIdx.x < ndkv)
+      bwd_dkv_body<D, NW, kModeBoth>(a, blockIdx.x);
+    else
+      bwd_dq_body<D, NW>(a, blockIdx.x - ndkv);
+  }
+}
+
+template <int D, int NP>
 constexpr size_t dkv_pair_smem_bytes() {
   return StageLayout<D, 3, 3 * 256>::kBytes + 2 * (size_t)NP * 2048;
 }
@@ -1068,42 +1125,20 @@ static int launch_dkv(const BwdArgs &a, hipStream_t st) {
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
 }
 
-// The dQ and the dK/dV kernels are independent, and each leaves part of the chip idle
-// while its last workgroups finish (a workgroup holds most of a CU's LDS, so the grid is
-// a small number of "rounds").  When a call runs both, one of them goes to a side
-// stream that is forked from and joined to the caller's stream by events, and the two
-// kernels' workgroups share the chip.  One side stream and event pair per device, made
-// on first use and kept; default priority; calls on one device take turns using them.
-struct SideStream {
-  hipStream_t stream = nullptr;
-  hipEvent_t fork = nullptr, join = nullptr;
-  std::mutex mu;
-  bool ok = false, tried = false;
-};
-static SideStream *side_stream() {
-  static SideStream per_device[64];
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
-  // BCATTN_SERIAL_BACKWARD=1 keeps the kernels on the caller's stream, one after the other
-  // (for profiling them apart)
+// BCATTN_SERIAL_BACKWARD=1 keeps the kernels apart, one launch each, one after the other (for
+// profiling them apart)
+static bool serial_backward() {
   static const bool serial = [] {
     const char *e = getenv("BCATTN_SERIAL_BACKWARD");
     return e != nullptr && e[0] == '1';
   }();
-  if (serial) return nullptr;
-  SideStream *ss = &per_device[dev];
-  std::lock_guard<std::mutex> lock(ss->mu);
-  if (!ss->tried) {
-    ss->tried = true;
-    ss->ok = hipStreamCreateWithFlags(&ss->stream, hipStreamNonBlocking) == hipSuccess &&
-             hipEventCreateWithFlags(&ss->fork, hipEventDisableTiming) == hipSuccess &&
-             hipEventCreateWithFlags(&ss->join, hipEventDisableTiming) == hipSuccess;
-  }
-  return ss->ok ? ss : nullptr;
+  return serial;
 }
 
-// NWQ: waves of the dQ kernel; NWK, SPLIT: waves of the dK/dV kernel and whether it
-// runs as two launches (dV, then dK).
+// NWQ: waves of the dQ kernel; NWK, SPLIT: waves of the single-wave dK/dV kernel and whether it
+// runs as two sets of workgroups (dV alone, dK alone); PAIRS > 0: the paired-wave dK/dV kernel.
+// A call that computes dQ and dK/dV runs them as one launch (see bwd_dkv_dq_kernel); a call for
+// one of them, or with BCATTN_SERIAL_BACKWARD=1, launches the kernels one by one on the given stream.
 template <int D, int NWQ, int NWK, bool SPLIT, int PAIRS = 0>
 static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
   if (!allow_dynamic_lds<&bwd_dq_kernel<D, NWQ>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
@@ -1113,45 +1148,41 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
     const int64_t rows = (int64_t)a.B * a.H * a.Sq_pad;
     hipLaunchKernelGGL(bwd_prep_kernel<D>, dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, a);
   }
+  const int R = a.G * a.Sq;
+  const unsigned ndq = xcd_grid((unsigned)((R + 32 * NWQ - 1) / (32 * NWQ) * a.Hkv * a.B));
+  const size_t smem_q = dq_smem_bytes<D>() + needed_table_bytes((a.Sk + 63) / 64);
+  constexpr int kKeysPerGroup = 32 * (PAIRS > 0 ? PAIRS : NWK);
+  const unsigned ndkv = xcd_grid((unsigned)((a.Sk + kKeysPerGroup - 1) / kKeysPerGroup * a.Hkv * a.B));
   const bool both = (a.stages & BCATTN_BWD_DQ) && (a.stages & BCATTN_BWD_DKV);
-  SideStream *ss = both ? side_stream() : nullptr;
-  std::unique_lock<std::mutex> turn;
-  hipStream_t kst = st;  // the other stream, when there is one
-  if (ss) {
-    turn = std::unique_lock<std::mutex>(ss->mu);
-    if (hipEventRecord(ss->fork, st) == hipSuccess && hipStreamWaitEvent(ss->stream, ss->fork, 0) == hipSuccess)
-      kst = ss->stream;
-    else
-      ss = nullptr;
+  if (both && !serial_backward()) {
+    if constexpr (PAIRS > 0) {
+      if (!allow_dynamic_lds<&bwd_dkv_dq_kernel<D, NWQ, PAIRS>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
+      if (!needed_table_fits(dkv_pair_smem_bytes<D, PAIRS>(), a.Sq_pad / 64)) return BCATTN_ERR_UNSUPPORTED;
+      const size_t smem_kv = dkv_pair_smem_bytes<D, PAIRS>() + needed_table_bytes(a.Sq_pad / 64);
+      hipLaunchKernelGGL((bwd_dkv_dq_kernel<D, NWQ, PAIRS>), dim3(ndkv + ndq), dim3(128 * PAIRS),
+                         smem_kv > smem_q ? smem_kv : smem_q, st, a, ndkv);
+    } else {
+      static_assert(NWQ == NWK, "both roles use the same workgroup size");
+      if (!allow_dynamic_lds<&bwd_dkv1_dq_kernel<D, NWQ, SPLIT>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
+      if (!needed_table_fits(dkv_smem_bytes<D>(), a.Sq_pad / 64)) return BCATTN_ERR_UNSUPPORTED;
+      const size_t smem_kv = dkv_smem_bytes<D>() + needed_table_bytes(a.Sq_pad / 64);
+      hipLaunchKernelGGL((bwd_dkv1_dq_kernel<D, NWQ, SPLIT>), dim3((SPLIT ? 2 : 1) * ndkv + ndq), dim3(64 * NWQ),
+                         smem_kv > smem_q ? smem_kv : smem_q, st, a, ndkv);
+    }
+    return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
   }
   int rc = BCATTN_OK;
-  // Work on the helper stream starts a little later than work on the caller's stream (it waits
-  // for the fork event).  A dK/dV grid that cannot fill the chip by itself goes first, on the
-  // caller's stream, and the dQ workgroups fill the CUs it leaves (4 % on the pi0.5 training
-  // shape); a larger one goes to the helper stream (1 % better on the others).
-  constexpr int kKeysPerGroup = 32 * (PAIRS > 0 ? PAIRS : NWK);
-  const bool dkv_first = (int64_t)((a.Sk + kKeysPerGroup - 1) / kKeysPerGroup) * a.Hkv * a.B < kSplitTarget;
-  const hipStream_t dkv_st = dkv_first ? st : kst, dq_st = dkv_first ? kst : st;
   if (a.stages & BCATTN_BWD_DKV) {
     if constexpr (PAIRS > 0) {
-      rc = launch_dkv_pair<D, PAIRS>(a, dkv_st);
+      rc = launch_dkv_pair<D, PAIRS>(a, st);
     } else if constexpr (SPLIT) {
-      if (!(rc = launch_dkv<D, NWK, kModeDV>(a, dkv_st))) rc = launch_dkv<D, NWK, kModeDK>(a, dkv_st);
+      if (!(rc = launch_dkv<D, NWK, kModeDV>(a, st))) rc = launch_dkv<D, NWK, kModeDK>(a, st);
     } else {
-      rc = launch_dkv<D, NWK, kModeBoth>(a, dkv_st);
+      rc = launch_dkv<D, NWK, kModeBoth>(a, st);
     }
   }
-  if (!rc && (a.stages & BCATTN_BWD_DQ)) {
-    const int R = a.G * a.Sq;
-    const int ntile_r = (R + 32 * NWQ - 1) / (32 * NWQ);
-    const size_t smem = dq_smem_bytes<D>() + needed_table_bytes((a.Sk + 63) / 64);
-    hipLaunchKernelGGL((bwd_dq_kernel<D, NWQ>), dim3(xcd_grid((unsigned)(ntile_r * a.Hkv * a.B))), dim3(64 * NWQ),
-                       smem, dq_st, a);
-  }
-  if (ss) {  // join, whatever happened in between: the caller's stream must not run ahead of the side stream
-    if (hipEventRecord(ss->join, ss->stream) != hipSuccess || hipStreamWaitEvent(st, ss->join, 0) != hipSuccess)
-      rc = rc ? rc : BCATTN_ERR_LAUNCH;
-  }
+  if (!rc && (a.stages & BCATTN_BWD_DQ))
+    hipLaunchKernelGGL((bwd_dq_kernel<D, NWQ>), dim3(ndq), dim3(64 * NWQ), smem_q, st, a);
   if (rc) return rc;
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
 }

@@ -113,6 +113,22 @@ __device__ __forceinline__ int xcd_item(unsigned id, unsigned n) {
   return (int)((id % kXcds) * chunk + id / kXcds);
 }
 
+// The kernel arguments reach a wave through scalar loads from a segment that nothing on the
+// CU has touched before; left to the compiler each group of arguments is fetched where it is first
+// needed, which makes a kernel's prologue a chain of dependent round trips to memory.  This reads
+// one word of every 64-byte line of the first BYTES of the segment in one go, so that the later
+// loads hit the scalar cache.  BYTES must not exceed the size of the explicit arguments.
+template <int BYTES>
+__device__ __forceinline__ void warm_kernel_arguments() {
+  typedef const __attribute__((address_space(4))) int kint;
+  kint *ka = (kint *)__builtin_amdgcn_kernarg_segment_ptr();
+  int x = 0;
+#pragma unroll
+  for (int i = 0; i < BYTES / 64; ++i) x |= ka[16 * i];
+  if (BYTES % 64) x |= ka[(BYTES - 4) / 4];
+  asm volatile("" ::"s"(x));
+}
+
 // ---------------------------------------------------------------------------
 // Kernel argument blocks (device pointers already offset to element 0).
 // ---------------------------------------------------------------------------

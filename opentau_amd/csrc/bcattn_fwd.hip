@@ -45,6 +45,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
 
   extern __shared__ __align__(1024) char smem[];
   __shared__ int red_s[2 * NW];
+  warm_kernel_arguments<sizeof(FwdArgs) + sizeof(SplitArgs)>();
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
@@ -126,14 +127,15 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
   // tiles are requested before anything is known about the rows (compute() skips a
   // tile that no row turns out to see).
   const int t_last = SPLIT ? min(nt_all, t_first + sp.tiles_per_split) : nt_all;
-  if (SPLIT) {
+  auto early_requests = [&]() __attribute__((always_inline)) {
     if (t_first < t_last) issue(t_first, StageC<0>{});
     if (t_first + 1 < t_last) issue(t_first + 1, StageC<1>{});
     if constexpr (NS >= 3)
       if (t_first + 2 < t_last) issue(t_first + 2, StageC<2>{});
     if constexpr (NS >= 4)
       if (t_first + 3 < t_last) issue(t_first + 3, StageC<3>{});
-  }
+  };
+  if (SPLIT) early_requests();
 
   // ---- this lane's query row ------------------------------------------------
   const int r = tile * BM + wave * 32 + n;
@@ -439,34 +441,57 @@ __global__ __launch_bounds__(256) void fwd_combine_kernel(const FwdArgs a, const
                     (db * 2 + rp) * 512 + 8 * lane;
   const int64_t po_step = (int64_t)ntile_r * (BM * D);
   float mx = -INFINITY;
-  for (int s0 = 0; s0 < sp.nsplit; s0 += CH) {
-    float mv[CH];
-#pragma unroll
-    for (int j = 0; j < CH; ++j) mv[j] = mlp[min(s0 + j, sp.nsplit - 1) * ml_step];
-#pragma unroll
-    for (int j = 0; j < CH; ++j) mx = fmaxf(mx, mv[j]);
-  }
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   float lsum = 0.f;
-  const float mref = mx == -INFINITY ? 0.f : mx;
-  for (int s0 = 0; s0 < sp.nsplit; s0 += CH) {
+  if (sp.nsplit <= CH) {
+    // the usual case: everything the thread needs is requested at once (one trip to memory)
     f32x2 ml[CH];
     e16x8 po[CH];
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
-      const int sj = min(s0 + j, sp.nsplit - 1);
+      const int sj = min(j, sp.nsplit - 1);
       ml[j] = *reinterpret_cast<const f32x2 *>(mlp + sj * ml_step);
       po[j] = *reinterpret_cast<const e16x8 *>(pp + sj * po_step);
     }
 #pragma unroll
+    for (int j = 0; j < CH; ++j) mx = fmaxf(mx, ml[j][0]);
+    const float mref = mx == -INFINITY ? 0.f : mx;
+#pragma unroll
     for (int j = 0; j < CH; ++j) {
-      // a split without a visible key has max -inf and sum 0: weight 0, not NaN;
-      // a partial is normalised by its own sum, so its weight carries that sum
-      const bool live = s0 + j < sp.nsplit && ml[j][0] != -INFINITY;
+      const bool live = j < sp.nsplit && ml[j][0] != -INFINITY;
       const float w = live ? fast_exp2((ml[j][0] - mref) * c) * ml[j][1] : 0.f;
       lsum += w;
 #pragma unroll
       for (int x = 0; x < 8; ++x) acc[x] += live ? w * (float)po[j][x] : 0.f;
+    }
+  } else {
+    for (int s0 = 0; s0 < sp.nsplit; s0 += CH) {
+      float mv[CH];
+#pragma unroll
+      for (int j = 0; j < CH; ++j) mv[j] = mlp[min(s0 + j, sp.nsplit - 1) * ml_step];
+#pragma unroll
+      for (int j = 0; j < CH; ++j) mx = fmaxf(mx, mv[j]);
+    }
+    const float mref = mx == -INFINITY ? 0.f : mx;
+    for (int s0 = 0; s0 < sp.nsplit; s0 += CH) {
+      f32x2 ml[CH];
+      e16x8 po[CH];
+#pragma unroll
+      for (int j = 0; j < CH; ++j) {
+        const int sj = min(s0 + j, sp.nsplit - 1);
+        ml[j] = *reinterpret_cast<const f32x2 *>(mlp + sj * ml_step);
+        po[j] = *reinterpret_cast<const e16x8 *>(pp + sj * po_step);
+      }
+#pragma unroll
+      for (int j = 0; j < CH; ++j) {
+        // a split without a visible key has max -inf and sum 0: weight 0, not NaN;
+        // a partial is normalised by its own sum, so its weight carries that sum
+        const bool live = s0 + j < sp.nsplit && ml[j][0] != -INFINITY;
+        const float w = live ? fast_exp2((ml[j][0] - mref) * c) * ml[j][1] : 0.f;
+        lsum += w;
+#pragma unroll
+        for (int x = 0; x < 8; ++x) acc[x] += live ? w * (float)po[j][x] : 0.f;
+      }
     }
   }
   const bool has = lsum > 0.f;

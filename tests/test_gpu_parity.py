@@ -605,7 +605,7 @@ def test_threads_with_their_own_streams_get_the_serial_results():
     give, bit for bit, what the same calls give one after the other."""
     import threading
 
-    b, sq, h, hkv, d = 2, 1100, 16, 2, 128  # long enough for the large-group kernels and the helper stream
+    b, sq, h, hkv, d = 2, 1100, 16, 2, 128  # long enough for the large-group kernels (dK/dV and dQ in one launch)
     ids = [g(t) for t in make_blocks(b, sq, "prefixlm", pad_tail=9)]
     cases = []
     for t in range(4):
@@ -686,8 +686,7 @@ def test_traced_graph_runs_the_same_kernels():
 def test_calls_replay_from_a_captured_graph():
     """A denoise step is many small calls; a caller that captures them in a HIP graph must get,
     on every replay, what the eager calls give for the inputs then in place (the library
-    allocates nothing and clears nothing; the backward's helper stream joins the capture through
-    its events).  Replays alternate with eager work and synchronisation."""
+    allocates nothing and clears nothing; every call stays on the captured stream).  Replays alternate with eager work and synchronisation."""
     b, sq, h, hkv, d, cross = 2, 50, 8, 1, 256, 200
     ids = [g(t) for t in make_blocks(b, sq, "prefixlm", cross=cross)]
     sids = [g(t) for t in make_blocks(b, 1100 // 8 + 3, "prefixlm", pad_tail=7)]
@@ -696,7 +695,7 @@ def test_calls_replay_from_a_captured_graph():
     kc, vc = g(randn((b, cross, hkv, d), torch.bfloat16, 2)), g(randn((b, cross, hkv, d), torch.bfloat16, 3))
     kn, vn = g(randn((b, sq, hkv, d), torch.bfloat16, 4)), g(randn((b, sq, hkv, d), torch.bfloat16, 5))
     s2 = sids[0].shape[1]
-    q2, k2, v2 = (g(t) for t in _qkv(b, s2, s2, 8, 1, 128, torch.bfloat16, seed=30))  # G*Sq >= 1024: two-stream backward
+    q2, k2, v2 = (g(t) for t in _qkv(b, s2, s2, 8, 1, 128, torch.bfloat16, seed=30))  # G*Sq >= 1024: the paired-wave backward
     go2 = g(randn((b, s2, 8, 128), torch.bfloat16, 37))
 
     def work():
@@ -705,7 +704,7 @@ def test_calls_replay_from_a_captured_graph():
         return (o1, o2, *fa.backward_raw(go2, q2, k2, v2, o2, lse2, *sids, 128**-0.5))
 
     side = torch.cuda.Stream()
-    with torch.cuda.stream(side):  # warm-up outside the capture (first calls set attributes, make the helper stream)
+    with torch.cuda.stream(side):  # warm-up outside the capture (first calls set kernel attributes)
         work()
     side.synchronize()
     graph = torch.cuda.CUDAGraph()
