@@ -14,12 +14,17 @@ from __future__ import annotations
 import torch
 
 from .flash_attn_hip import (
+    BlockIds,
     flash_attn_blockmask,
     flash_attn_blockmask_kvcache,
     make_att_block_ids,
 )
 
 ATTENTION_IMPLEMENTATION = "flash_hip"
+
+
+def _held(attention_block_ids) -> BlockIds | None:
+    return attention_block_ids if isinstance(attention_block_ids, BlockIds) else None
 
 
 def flash_hip_active(attention_implementation: str) -> bool:
@@ -39,7 +44,8 @@ def build_attention_inputs(
     Counterpart of ``build_attention_inputs`` in
     ``src/opentau/policies/pi07_paligemma/low_level/modeling_pi07_low_level.py:257-275``.
     With ``use_flash`` the dense mask is never built and ``attention_mask`` is
-    ``None``.  Without it this backend has nothing to offer: the dense-mask
+    ``None``.  The block ids come as a :class:`BlockIds`, which unpacks like the reference's tuple and
+    lets the calls below prepare the kernels' view of the mask once for all layers.  Without it this backend has nothing to offer: the dense-mask
     backends belong to the caller, so it raises.
     """
     if not use_flash:
@@ -47,7 +53,7 @@ def build_attention_inputs(
             "build_attention_inputs(use_flash=False): the dense-mask backends (eager, sdpa) are the "
             "caller's; this package only serves the block-id backend"
         )
-    return None, make_att_block_ids(pad_masks, att_masks, n_cross_att_tokens, cross_att_pad_masks)
+    return None, BlockIds(*make_att_block_ids(pad_masks, att_masks, n_cross_att_tokens, cross_att_pad_masks))
 
 
 def flash_attention_forward(
@@ -70,7 +76,8 @@ def flash_attention_forward(
     """
     q_blk, k_blk, q_valid, k_valid = attention_block_ids
     scale = scaling if scaling is not None else head_dim**-0.5
-    out = flash_attn_blockmask(query_states, key_states, value_states, q_blk, k_blk, q_valid, k_valid, scale)
+    out = flash_attn_blockmask(query_states, key_states, value_states, q_blk, k_blk, q_valid, k_valid, scale,
+                               block_ids=_held(attention_block_ids))
     return out.reshape(batch_size, out.shape[1], -1)
 
 
@@ -98,7 +105,7 @@ def flash_attention_forward_kvcache(
     scale = scaling if scaling is not None else head_dim**-0.5
     out = flash_attn_blockmask_kvcache(
         query_states, cache_key_states, cache_value_states, key_states, value_states, q_blk, k_blk, q_valid,
-        k_valid, scale,
+        k_valid, scale, block_ids=_held(attention_block_ids),
     )
     return out.reshape(batch_size, out.shape[1], -1)
 
@@ -120,7 +127,8 @@ def attend_bhsd(
     q_blk, k_blk, q_valid, k_valid = attention_block_ids
     scale = scaling if scaling is not None else q.shape[-1] ** -0.5
     out = flash_attn_blockmask(
-        q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), q_blk, k_blk, q_valid, k_valid, scale
+        q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), q_blk, k_blk, q_valid, k_valid, scale,
+        block_ids=_held(attention_block_ids),
     )
     return out.reshape(out.shape[0], out.shape[1], -1)
 
@@ -141,6 +149,6 @@ def attend_bhsd_kvcache(
     ck, cv = cached_kv
     out = flash_attn_blockmask_kvcache(
         q.transpose(1, 2), ck.transpose(1, 2), cv.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2),
-        q_blk, k_blk, q_valid, k_valid, scale,
+        q_blk, k_blk, q_valid, k_valid, scale, block_ids=_held(attention_block_ids),
     )
     return out.reshape(out.shape[0], out.shape[1], -1)

@@ -27,6 +27,7 @@ from . import _loader
 from ._loader import is_available, load_error
 
 __all__ = [
+    "BlockIds",
     "INT_BLK_MIN",
     "flash_attn_blockmask",
     "flash_attn_blockmask_kvcache",
@@ -78,6 +79,50 @@ def make_att_block_ids(
     k_blk = torch.cat([cross, blk], dim=1)
     k_valid = torch.cat([cross_att_pad_masks.to(torch.bool), valid], dim=1)
     return blk, k_blk, valid, k_valid
+
+
+class BlockIds(tuple):
+    """``(q_blk, k_blk, q_valid, k_valid)`` that also carries the kernels' workspace for this mask.
+
+    A policy builds one mask per forward pass and hands the same block ids to every layer
+    (``src/opentau/policies/pi05/paligemma_with_expert.py:758-768``, once per layer).  The kernels
+    fold the ids into per-tile summaries before they run; a plain tuple makes every layer call
+    allocate a workspace and repeat that pass.  Calls that are given a ``BlockIds`` keep the workspace
+    here, compute the summaries on the first call only, and the backward of each layer finds the
+    forward's key summary (and, from the second layer on, its own query summary) in place.
+
+    It unpacks like the plain tuple (``q_blk, k_blk, q_valid, k_valid = ids``).  The summaries are tied
+    to the id tensors' storage, shape and version counter: an in-place edit of an id tensor is seen
+    and the summaries are computed again.  One ``BlockIds`` serves one stream at a time (calls on it
+    share the workspace).
+    """
+
+    def __new__(cls, q_blk, k_blk, q_valid, k_valid):
+        q_blk, q_valid = _ids(q_blk, q_valid)
+        k_blk, k_valid = _ids(k_blk, k_valid)
+        self = super().__new__(cls, (q_blk, k_blk, q_valid, k_valid))
+        self._slots = {}
+        return self
+
+    def _stamp(self):
+        return tuple((t.data_ptr(), t._version, tuple(t.shape)) for t in self)
+
+    def _slot(self, key, need: int, device):
+        """The workspace slot of one kind of call, at least ``need`` bytes; its ``fwd`` / ``bwd`` flags say
+        which summaries it already holds for the ids as they are now."""
+        stamp = self._stamp()
+        slot = self._slots.get(key)
+        if slot is None or slot["ws"].numel() < need or slot["ws"].device != device:
+            slot = {"ws": torch.empty(max(need, 16), dtype=torch.uint8, device=device), "fwd": False, "bwd": False}
+            self._slots[key] = slot
+        if slot.get("stamp") != stamp:
+            slot["stamp"], slot["fwd"], slot["bwd"] = stamp, False, False
+        return slot
+
+
+def as_block_ids(ids) -> BlockIds:
+    """``ids`` itself when it already is a :class:`BlockIds`, else one made from the four tensors."""
+    return ids if isinstance(ids, BlockIds) else BlockIds(*ids)
 
 
 # --------------------------------------------------------------------------- #
@@ -182,6 +227,7 @@ def forward_raw(
     out: torch.Tensor | None = None,
     want_lse: bool = True,
     static_scratch: bool = False,
+    block_ids: BlockIds | None = None,
 ):
     """One forward through the C ABI.  Returns ``(out (B,Sq,H,D), lse (B,H,Sq) | None)``.
 
@@ -193,17 +239,21 @@ def forward_raw(
     sampling (``src/opentau/policies/candidates.py:114-127``).  ``static_scratch`` (with
     ``kvcache``) takes ``bcattn_fwd_kvcache_static``: the library's own fixed scratch instead of
     a workspace, so that the call itself allocates nothing when ``out`` is given and
-    ``want_lse`` is off.
+    ``want_lse`` is off.  ``block_ids`` (the :class:`BlockIds` the four id tensors came from) keeps
+    the workspace and the summaries for the next call with the same mask.
     """
     lib = _loader.require_library()
     _check_inputs(q, k, v)
     extra = _head_dim_padding(q)
+    if block_ids is not None and (workspace is not None or static_scratch):
+        raise RuntimeError("block_ids brings its own workspace")
     if static_scratch and (extra or not kvcache or workspace is not None):
         raise RuntimeError("static_scratch goes with kvcache=True, no workspace and a head_dim the kernels take")
     if extra:
         o, lse = forward_raw(_padded(q, extra), _padded(k, extra), _padded(v, extra), q_blk, k_blk, q_valid, k_valid,
                              scale, _padded(k_new, extra), _padded(v_new, extra), kvcache=kvcache,
-                             workspace=workspace, summary_ready=summary_ready, want_lse=want_lse)
+                             workspace=workspace, summary_ready=summary_ready, want_lse=want_lse,
+                             block_ids=block_ids)
         o = o[..., : q.shape[-1]]
         return (o.contiguous() if out is None else out.copy_(o)), lse
     code, vec = _DTYPES[q.dtype]
@@ -239,6 +289,14 @@ def forward_raw(
         return out, lse
     size_fn = lib.bcattn_fwd_kvcache_workspace_bytes if kvcache else lib.bcattn_fwd_workspace_bytes
     need = size_fn(ctypes.byref(p))
+    slot = None
+    if block_ids is not None:
+        if sk1 == 0:  # plain self-attention: the backward's workspace starts with the same key summary
+            key, need = ("self", b, sq, sk0), max(need, _bwd_workspace_bytes(lib, b, sq, sk0, h, hkv, d, code))
+        else:
+            key = ("two", kvcache, b, sq, sk0, sk1, h, hkv, d, share)
+        slot = block_ids._slot(key, need, q.device)
+        workspace, p.summary_ready = slot["ws"], 1 if slot["fwd"] else 0
     if workspace is None or workspace.numel() < need:
         if summary_ready:
             raise RuntimeError("summary_ready needs the workspace of the earlier call")
@@ -247,7 +305,15 @@ def forward_raw(
     with torch.cuda.device(q.device):
         fn = lib.bcattn_fwd_kvcache if kvcache else lib.bcattn_fwd
         _check(fn(ctypes.byref(p), _stream(q.device)), lib)
+    if slot is not None:
+        slot["fwd"] = True
     return out, lse
+
+
+def _bwd_workspace_bytes(lib, b, sq, sk, h, hkv, d, code) -> int:
+    p = _loader.BwdParams()
+    p.B, p.Sq, p.Sk, p.H, p.Hkv, p.D, p.dtype = b, sq, sk, h, hkv, d, code
+    return int(lib.bcattn_bwd_workspace_bytes(ctypes.byref(p)))
 
 
 def kvcache_workspace_bytes(b: int, sq: int, sk0: int, sk1: int, h: int, hkv: int, d: int,
@@ -261,11 +327,13 @@ def kvcache_workspace_bytes(b: int, sq: int, sk0: int, sk1: int, h: int, hkv: in
 
 
 def backward_raw(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale: float, *, stages: int = 0,
-                 workspace: torch.Tensor | None = None, summary_ready: bool = False, grads=None):
+                 workspace: torch.Tensor | None = None, summary_ready: bool = False, grads=None,
+                 block_ids: BlockIds | None = None):
     """One backward through the C ABI.  Returns ``(dq, dk, dv)``.
 
     ``stages`` selects parts (``_loader.BWD_DELTA | BWD_DQ | BWD_DKV``; 0 = all); parts
-    run separately must share ``workspace`` (and ``grads``, the output triple).
+    run separately must share ``workspace`` (and ``grads``, the output triple).  ``block_ids``: as for
+    :func:`forward_raw`; the workspace it keeps already holds the forward's key summary.
     """
     lib = _loader.require_library()
     _check_inputs(q, k, v)
@@ -273,7 +341,8 @@ def backward_raw(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale
     if extra:
         d = q.shape[-1]
         got = backward_raw(*(_padded(t, extra) for t in (d_out, q, k, v, out)), lse, q_blk, k_blk, q_valid, k_valid,
-                           scale, stages=stages, workspace=workspace, summary_ready=summary_ready)
+                           scale, stages=stages, workspace=workspace, summary_ready=summary_ready,
+                           block_ids=block_ids)
         got = tuple(t[..., :d] for t in got)
         if grads is not None:
             return tuple(dst.copy_(src) for dst, src in zip(grads, got))
@@ -301,6 +370,12 @@ def backward_raw(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale
     p.dtype, p.scale = code, float(scale)
     p.stages, p.summary_ready = int(stages), 1 if summary_ready else 0
     need = lib.bcattn_bwd_workspace_bytes(ctypes.byref(p))
+    slot = None
+    if block_ids is not None:
+        if workspace is not None:
+            raise RuntimeError("block_ids brings its own workspace")
+        slot = block_ids._slot(("self", b, sq, sk), need, q.device)
+        workspace, p.summary_ready = slot["ws"], 1 if slot["bwd"] else 0
     if workspace is None or workspace.numel() < need:
         if summary_ready or (stages and not stages & _loader.BWD_DELTA):
             raise RuntimeError("this call needs the workspace an earlier call filled")
@@ -308,6 +383,8 @@ def backward_raw(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale
     p.workspace, p.workspace_bytes = workspace.data_ptr(), workspace.numel()
     with torch.cuda.device(q.device):
         _check(lib.bcattn_bwd(ctypes.byref(p), _stream(q.device)), lib)
+    if slot is not None:
+        slot["fwd"] = slot["bwd"] = True  # the backward's summary pass covers the keys as well
     return dq, dk, dv
 
 
@@ -373,12 +450,13 @@ def _op_bwd(
     q_valid: torch.Tensor,
     k_valid: torch.Tensor,
     scale: float,
+    stages: int = 0,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    return backward_raw(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale)
+    return backward_raw(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale, stages=stages)
 
 
 @_op_bwd.register_fake
-def _(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale):
+def _(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale, stages=0):
     return (
         q.new_empty(q.shape),
         k.new_empty(k.shape),
@@ -393,10 +471,19 @@ def _fwd_setup(ctx, inputs, output):
     ctx.scale = scale
 
 
+def _wanted_stages(want_q: bool, want_kv: bool) -> int:
+    """The parts of the backward somebody asks for (the row sums always).  With K and V detached
+    (knowledge insulation, ``src/opentau/policies/pi05/modeling_pi05.py:1752-1757``) the dK/dV kernel,
+    the longer of the two, is not launched."""
+    return _loader.BWD_DELTA | (_loader.BWD_DQ if want_q else 0) | (_loader.BWD_DKV if want_kv else 0)
+
+
 def _fwd_backward(ctx, d_out, _d_lse):
     q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid = ctx.saved_tensors
-    dq, dk, dv = _op_bwd(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, ctx.scale)
-    return dq, dk, dv, None, None, None, None, None
+    need = ctx.needs_input_grad
+    stages = _wanted_stages(need[0], need[1] or need[2])
+    dq, dk, dv = _op_bwd(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, ctx.scale, stages)
+    return dq if need[0] else None, dk if need[1] else None, dv if need[2] else None, None, None, None, None, None
 
 
 _op_fwd.register_autograd(_fwd_backward, setup_context=_fwd_setup)
@@ -410,18 +497,27 @@ def _kvc_setup(ctx, inputs, output):
 
 
 def _kvc_backward(ctx, d_out, _d_lse):
+    # The backward kernels take the keys as one segment, so the two are joined here: a copy of
+    # B*Sk*Hkv*D elements per layer, against attention work that grows with Sq*Sk*H*D.  (Training
+    # with a cache is the knowledge-insulation case, whose cached K/V are detached: then only dQ
+    # and the new keys' gradients are wanted, and with nothing wanted for K/V the dK/dV kernel is skipped.)
     q, k_cache, v_cache, k_new, v_new, out, lse, q_blk, k_blk, q_valid, k_valid = ctx.saved_tensors
+    need = ctx.needs_input_grad
     n0 = k_cache.shape[1]
     share = q.shape[0] // k_cache.shape[0]
     if share > 1:  # a shared cache entry collects the gradients of all the entries that read it
         k_cache, v_cache = (t.repeat_interleave(share, dim=0) for t in (k_cache, v_cache))
     k = torch.cat([k_cache, k_new], dim=1)
     v = torch.cat([v_cache, v_new], dim=1)
-    dq, dk, dv = _op_bwd(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, ctx.scale)
-    dkc, dvc = dk[:, :n0], dv[:, :n0]
-    if share > 1:
-        dkc, dvc = (t.reshape(-1, share, *t.shape[1:]).float().sum(1).to(t.dtype) for t in (dkc, dvc))
-    return dq, dkc, dvc, dk[:, n0:], dv[:, n0:], None, None, None, None, None
+    stages = _wanted_stages(need[0], any(need[1:5]))
+    dq, dk, dv = _op_bwd(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, ctx.scale, stages)
+    dkc = dvc = None
+    if need[1] or need[2]:
+        dkc, dvc = dk[:, :n0], dv[:, :n0]
+        if share > 1:
+            dkc, dvc = (t.reshape(-1, share, *t.shape[1:]).float().sum(1).to(t.dtype) for t in (dkc, dvc))
+    return (dq if need[0] else None, dkc if need[1] else None, dvc if need[2] else None,
+            dk[:, n0:] if need[3] else None, dv[:, n0:] if need[4] else None, None, None, None, None, None)
 
 
 _op_fwd_kvcache.register_autograd(_kvc_backward, setup_context=_kvc_setup)
@@ -429,6 +525,31 @@ _op_fwd_kvcache.register_autograd(_kvc_backward, setup_context=_kvc_setup)
 
 def _needs_graph(*ts: torch.Tensor) -> bool:
     return torch.compiler.is_compiling() or (torch.is_grad_enabled() and any(t.requires_grad for t in ts))
+
+
+class _HeldBlockMask(torch.autograd.Function):
+    """The eager autograd path of calls that come with a :class:`BlockIds`: forward and backward go
+    through the raw calls with the holder's workspace, so the tile summaries are made once per mask,
+    not once per layer and direction (the traced path, ``bcattn::fwd`` / ``bcattn::bwd``, carries no
+    Python object and makes them per call).  Gradients that nobody asks for are not computed: with K and
+    V detached (knowledge insulation, ``src/opentau/policies/pi05/modeling_pi05.py:1752-1757``) the
+    dK/dV kernel is skipped."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, scale, held):
+        out, lse = forward_raw(q, k, v, *held, scale, block_ids=held)
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.scale, ctx.held = scale, held
+        return out
+
+    @staticmethod
+    def backward(ctx, d_out):
+        q, k, v, out, lse = ctx.saved_tensors
+        want_q, want_kv = ctx.needs_input_grad[0], ctx.needs_input_grad[1] or ctx.needs_input_grad[2]
+        stages = _loader.BWD_DELTA | (_loader.BWD_DQ if want_q else 0) | (_loader.BWD_DKV if want_kv else 0)
+        dq, dk, dv = backward_raw(d_out, q, k, v, out, lse, *ctx.held, ctx.scale, stages=stages, block_ids=ctx.held)
+        return (dq if want_q else None, dk if ctx.needs_input_grad[1] else None,
+                dv if ctx.needs_input_grad[2] else None, None, None)
 
 
 def flash_attn_blockmask(
@@ -440,14 +561,21 @@ def flash_attn_blockmask(
     q_valid: torch.Tensor,
     k_valid: torch.Tensor,
     scale: float,
+    *,
+    block_ids: BlockIds | None = None,
 ) -> torch.Tensor:
     """Block-causal flash attention, ``(B,Sq,H,D), (B,Sk,Hkv,D) x2 -> (B,Sq,H,D)``.
 
     Same signature and semantics as the reference's ``flash_attn_blockmask``
     (``src/opentau/policies/flash_attn_cuda/__init__.py:146-171``).  Rows with no
     visible key come back as zeros.  Raises ``RuntimeError`` when the kernels are
-    unavailable.
+    unavailable.  ``block_ids``: the :class:`BlockIds` the four id tensors were unpacked from, when
+    there is one; its workspace then serves this call (and its backward).
     """
+    if block_ids is not None and not torch.compiler.is_compiling():
+        if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
+            return _HeldBlockMask.apply(q, k, v, float(scale), block_ids)
+        return forward_raw(q, k, v, *block_ids, scale, want_lse=False, block_ids=block_ids)[0]
     if _needs_graph(q, k, v):
         return _op_fwd(q, k, v, q_blk, k_blk, q_valid, k_valid, float(scale))[0]
     return forward_raw(q, k, v, q_blk, k_blk, q_valid, k_valid, scale, want_lse=False)[0]
@@ -464,6 +592,8 @@ def flash_attn_blockmask_kvcache(
     q_valid: torch.Tensor,
     k_valid: torch.Tensor,
     scale: float,
+    *,
+    block_ids: BlockIds | None = None,
 ) -> torch.Tensor:
     """Attention of a few query rows over ``[k_cache ; k_new]`` without the concat.
 
@@ -478,6 +608,9 @@ def flash_attn_blockmask_kvcache(
     the ``n`` copies of the prefix cache that ``expand_kv_cache`` makes
     (``src/opentau/policies/candidates.py:114-127``).
     """
+    if block_ids is not None and not _needs_graph(q, k_cache, v_cache, k_new, v_new):
+        return forward_raw(q, k_cache, v_cache, *block_ids, scale, k_new, v_new, kvcache=True, want_lse=False,
+                           block_ids=block_ids)[0]
     if _needs_graph(q, k_cache, v_cache, k_new, v_new):
         return _op_fwd_kvcache(q, k_cache, v_cache, k_new, v_new, q_blk, k_blk, q_valid, k_valid, float(scale))[0]
     return forward_raw(

@@ -29,8 +29,7 @@ class StaticKVCache:
         self.k = torch.empty(shape, dtype=dtype, device=device)
         self.v = torch.empty(shape, dtype=dtype, device=device)
         self.length = 0
-        self._ids = None        # the block ids whose summary the workspace holds
-        self._workspace = None
+        self._held = None  # the BlockIds (ids + workspace with their summary) of the mask in use
 
     @property
     def n_layers(self) -> int:
@@ -62,7 +61,7 @@ class StaticKVCache:
     def reset(self) -> None:
         """Forget the rows and the mask summary (a new observation; or block ids that were changed in place)."""
         self.length = 0
-        self._ids = None
+        self._held = None
 
     def layer(self, layer: int) -> tuple[torch.Tensor, torch.Tensor]:
         """The valid rows of a layer, ``(B, length, Hkv, D)`` views."""
@@ -78,25 +77,29 @@ class StaticKVCache:
         ``q (B*n, Sq, H, D)`` over ``[cache[layer] ; k, v (B*n, Sq, Hkv, D)]`` -> ``(B*n, Sq, H*D)``.
 
         ``attention_block_ids`` cover the concatenation (``make_att_block_ids(pad, att, n_cross, cross_pad)``).
-        The same tuple object passed again (every layer and denoise step does) reuses the key-tile summary.
-        ``n > 1``: candidates of best-of-N sampling, in ``(b n)`` order, share cache entry ``b``.  Inference
-        only.
+        Every layer and denoise step passes the same ids: their tile summary is made on the first call
+        and reused for as long as the id tensors stay what they were (same storage, shape and version
+        counter: an in-place edit is seen, and the summary is made again).  A :class:`BlockIds`
+        is used as it is.  ``n > 1``: candidates of best-of-N sampling, in ``(b n)`` order, share cache
+        entry ``b``.  Inference only.
         """
-        q_blk, k_blk, q_valid, k_valid = attention_block_ids
+        held = self._hold(attention_block_ids)
         scale = scaling if scaling is not None else query_states.shape[-1] ** -0.5
         kc, vc = self.layer(layer)
-        ready = self._ids is attention_block_ids and self._workspace is not None
-        if not ready:
-            self._workspace = self._sized_workspace(query_states, kc, key_states)
-        out, _ = fa.forward_raw(query_states, kc, vc, q_blk, k_blk, q_valid, k_valid, scale, key_states, value_states,
-                                kvcache=True, workspace=self._workspace, summary_ready=ready, want_lse=False)
-        self._ids = attention_block_ids
+        out, _ = fa.forward_raw(query_states, kc, vc, *held, scale, key_states, value_states, kvcache=True,
+                                want_lse=False, block_ids=held)
         return out.reshape(out.shape[0], out.shape[1], -1)
 
-    def _sized_workspace(self, q, kc, k_new) -> torch.Tensor:
-        need = fa.kvcache_workspace_bytes(q.shape[0], q.shape[1], kc.shape[1], k_new.shape[1], q.shape[2], kc.shape[2],
-                                          q.shape[3], q.dtype)
-        ws = self._workspace
-        if ws is None or ws.numel() < need or ws.device != q.device:
-            ws = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
-        return ws
+    def _hold(self, ids) -> fa.BlockIds:
+        if isinstance(ids, fa.BlockIds):
+            return ids
+        held = self._held
+        # the caller's own tensors, unchanged since last time (same objects, same version counters),
+        # mean the same mask: the holder made from them then still stands
+        source = tuple((t, t._version) for t in ids)
+        if (held is None or len(source) != len(held._source)
+                or any(a is not b or va != vb for (a, va), (b, vb) in zip(source, held._source))):
+            held = fa.BlockIds(*ids)
+            held._source = source
+            self._held = held
+        return held

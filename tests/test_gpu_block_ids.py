@@ -1,0 +1,123 @@
+"""``BlockIds``: the mask's tile summaries are made once per forward pass, not once per layer.
+
+The reference hands the same ``attention_block_ids`` to every layer's ``flash_attention_forward``
+(``src/opentau/policies/pi05/paligemma_with_expert.py:758-768``).  Here the holder keeps the kernels'
+workspace; these tests check, through the model-facing calls, that later layers (and every backward)
+reuse the first call's summary, that the results are bit-identical to calls without a holder, and that
+an in-place edit of the ids is noticed.
+"""
+
+import pytest
+import torch
+
+from opentau_amd import attention
+from opentau_amd import flash_attn_hip as fa
+from opentau_amd.kv_cache import StaticKVCache
+
+from helpers import make_blocks, randn
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _need_kernels():
+    if not torch.cuda.is_available():
+        pytest.skip("needs a GPU")
+    if not fa.is_available():
+        raise RuntimeError(f"HIP kernels unavailable on a GPU box: {fa.load_error()}")
+
+
+def g(t):
+    return t.to(DEV)
+
+
+def _layer_inputs(layer, b, s, h, hkv, d, dtype=torch.bfloat16):
+    return (g(randn((b, s, h, d), dtype, 100 + layer)), g(randn((b, s, hkv, d), dtype, 200 + layer)),
+            g(randn((b, s, hkv, d), dtype, 300 + layer)), g(randn((b, s, h * d), dtype, 400 + layer)))
+
+
+@pytest.mark.parametrize("head_dim,heads", [(128, 16), (256, 8)])
+def test_layers_share_one_summary_and_match_the_plain_calls(head_dim, heads):
+    b, s, hkv, layers = 2, 300, 2, 4
+    plain = tuple(g(t) for t in make_blocks(b, s, "prefixlm", pad_tail=17))
+    _, held = attention.build_attention_inputs(True, *_pad_att(b, s))
+    assert isinstance(held, fa.BlockIds) and all(torch.equal(a, c) for a, c in zip(held, plain))
+    for layer in range(layers):
+        q, k, v, go = _layer_inputs(layer, b, s, heads, hkv, head_dim)
+        got, want = [], []
+        for ids, res in ((held, got), (plain, want)):
+            qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+            out = attention.flash_attention_forward(None, ids, b, head_dim, qq, kk, vv)
+            out.backward(go)
+            res += [out.detach(), qq.grad, kk.grad, vv.grad]
+        torch.cuda.synchronize()
+        for name, a, c in zip(("out", "dq", "dk", "dv"), got, want):
+            assert torch.equal(a, c), f"layer {layer}: {name} differs from the call without a holder"
+    slot = held._slots[("self", b, s, s)]
+    assert slot["fwd"] and slot["bwd"] and len(held._slots) == 1  # one workspace served every call
+
+
+def _pad_att(b, s, pad_tail=17):
+    pad = torch.ones(b, s, dtype=torch.bool)
+    pad[0, -pad_tail:] = False
+    att = torch.zeros(b, s, dtype=torch.int32)
+    att[:, s // 2:] = 1
+    return g(pad), g(att)
+
+
+def test_summary_is_not_made_again_until_the_ids_change():
+    """The forward kernel sees the keys' ids and validity only through the summary pass.  Memory
+    changed behind the version counter (``.data``) therefore changes nothing while the summary is
+    reused; an ordinary in-place edit bumps the counter, and the next call summarises again."""
+    b, s, h, hkv, d = 2, 200, 8, 1, 256
+    _, ids = attention.build_attention_inputs(True, *_pad_att(b, s))
+    held = fa.BlockIds(ids[0], ids[1].clone(), ids[2], ids[3].clone())  # (self-attention shares the q / k tensors)
+    original = tuple(t.clone() for t in held)
+    q, k, v, _ = _layer_inputs(0, b, s, h, hkv, d)
+    first = attention.flash_attention_forward(None, held, b, d, q, k, v)
+    held[3].data[:, : s // 2] = False  # invisible to the version counter
+    again = attention.flash_attention_forward(None, held, b, d, q, k, v)
+    assert torch.equal(again, first), "the summary was computed again although the ids' version did not change"
+    held[3].data.copy_(original[3])
+    held[3][:, : s // 4] = False  # an in-place edit the holder can see
+    edited = attention.flash_attention_forward(None, held, b, d, q, k, v)
+    want = attention.flash_attention_forward(None, tuple(t.clone() for t in held), b, d, q, k, v)
+    torch.cuda.synchronize()
+    assert torch.equal(edited, want) and not torch.equal(edited, first)
+
+
+def test_detached_keys_skip_the_key_gradients():
+    b, s, h, hkv, d = 2, 150, 8, 1, 256
+    _, held = attention.build_attention_inputs(True, *_pad_att(b, s))
+    q, k, v, go = _layer_inputs(1, b, s, h, hkv, d)
+    qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+    attention.flash_attention_forward(None, held, b, d, qa, ka, va).backward(go)
+    qd = q.clone().requires_grad_(True)
+    attention.flash_attention_forward(None, held, b, d, qd, k, v).backward(go)  # K, V detached
+    qp = q.clone().requires_grad_(True)
+    attention.flash_attention_forward(None, tuple(held), b, d, qp, k, v).backward(go)  # the traced ops' path
+    torch.cuda.synchronize()
+    assert torch.equal(qd.grad, qa.grad) and torch.equal(qp.grad, qa.grad)
+
+
+def test_static_cache_notices_edited_ids():
+    layers, b, sq, h, hkv, d, cross = 2, 2, 50, 8, 1, 256, 300
+    cache = StaticKVCache(layers, b, cross, hkv, d, device=DEV)
+    for layer in range(layers):
+        cache.fill(layer, g(randn((b, cross, hkv, d), torch.bfloat16, 10 + layer)),
+                   g(randn((b, cross, hkv, d), torch.bfloat16, 20 + layer)))
+    ids = tuple(g(t) for t in make_blocks(b, sq, "prefixlm", cross=cross))
+    q, kn, vn = (g(randn((b, sq, hh, d), torch.bfloat16, 30 + n)) for n, hh in enumerate((h, hkv, hkv)))
+
+    def fresh(layer):
+        kc, vc = cache.layer(layer)
+        o, _ = fa.forward_raw(q, kc, vc, *ids, d**-0.5, kn, vn, kvcache=True)
+        return o.reshape(b, sq, -1)
+
+    assert torch.equal(cache.attend(0, q, kn, vn, ids), fresh(0))
+    held = cache._held
+    assert torch.equal(cache.attend(1, q, kn, vn, ids), fresh(1)) and cache._held is held  # same mask: reused
+    ids[3][1, 100:200] = False  # a new observation written into the same buffers
+    assert torch.equal(cache.attend(0, q, kn, vn, ids), fresh(0)) and cache._held is not held
+    torch.cuda.synchronize()
