@@ -5,12 +5,16 @@ One step = one forward + backward of the cosmos3-shape attention call (bf16, B4
 H64 Hkv8 D128, S = 4352 prefix + 50 action tokens, seeded synthetic inputs)
 through the C ABI.  ``value`` is TFLOP/s on unmasked FLOPs only
 (``14 * D * H * pairs`` per step: 4 for the forward's two products, 10 for the
-backward's five), inputs resident in HBM.  Every part of the step is bracketed
-by HIP events on the launch stream inside the timed region, which gives the
-per-kernel durations behind ``roofline``.  The pi0.5 denoise attention (18
-prefix calls + 180 cached-suffix calls at B=8) is timed after it and reported
-under ``denoise``.  ``cpu_baseline`` is the eager CPU oracle on a bounded slice
-of the same workload.
+backward's five), inputs resident in HBM, from the wall clock around exactly
+``--steps`` steps; HIP events around every step give the median and the minimum
+beside it.  Every part of the step is then launched alone between HIP events on
+the launch stream, which gives the per-kernel durations behind ``roofline``.
+``other_workloads`` holds the same record for the two head_dim 256 training shapes
+(pi0.5, pi0.6); ``dispatch`` times the PyTorch-facing op (autograd, allocation of
+the outputs) beside the raw C-ABI step; ``denoise`` the pi0.5 inference attention
+(18 prefix calls + 180 cached-suffix calls at B=8) and pi0.6's (34 x 5 suffix
+calls at B=16); ``cpu_baseline`` is the eager CPU oracle on a bounded slice of
+the headline workload, in the workload's own dtype.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-denoise]
 """
@@ -20,22 +24,40 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import re
+import statistics
 import sys
 import time
+from pathlib import Path
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0
+ROOT = Path(__file__).resolve().parent
 
 
-# HBM bytes per launch (fetched + written) of the kernels of the default workload, from two
-# counter runs (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what
-# the same counter reads for a plain 1 GiB device copy (FETCH_SIZE reads half the bytes: factor 2.0;
-# WRITE_SIZE: factor 1.0).  Other workloads have no such measurement and report null.
-HBM_TRAFFIC_BYTES = {
-    ("c5", "fwd"): int((286503.7 * 2.0 + 286134.8) * 1024),
-    ("c5", "bwd_dq"): int((437434.9 * 2.0 + 281728.0) * 1024),
-    ("c5", "bwd_dkv"): int((675657.6 * 2.0 + 70432.0) * 1024),
-}
+def hbm_traffic_from_profile(workload: str) -> dict:
+    """HBM bytes per launch of a workload's kernels from the tracked counter summary
+    (``profiles/hbm_traffic_counters.txt``: rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, KiB per
+    dispatch, each scaled by what the same counter reads for a plain device copy of known size;
+    the file states the commands and the two factors).  Not a measurement of this run: the record
+    says so (``traffic_source``); parts the file does not cover give ``None``."""
+    path = ROOT / "profiles" / "hbm_traffic_counters.txt"
+    out = {}
+    if not path.exists():
+        return out
+    scale = {"FETCH_SIZE": 1.0, "WRITE_SIZE": 1.0}
+    rows = []
+    for line in path.read_text().splitlines():
+        m = re.match(r"^scale\s+(FETCH_SIZE|WRITE_SIZE)\s+([0-9.]+)", line)
+        if m:
+            scale[m.group(1)] = float(m.group(2))
+        m = re.match(r"^traffic\s+(\w+)\s+(\w+)\s+FETCH_SIZE_KiB\s+([0-9.]+)\s+WRITE_SIZE_KiB\s+([0-9.]+)", line)
+        if m:
+            rows.append(m.groups())
+    for wl, part, fetch, write in rows:
+        if wl == workload:
+            out[part] = int((float(fetch) * scale["FETCH_SIZE"] + float(write) * scale["WRITE_SIZE"]) * 1024)
+    return out
 
 
 def main() -> int:
@@ -44,10 +66,10 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-denoise", action="store_true", help="skip the pi0.5 denoise leg")
+    ap.add_argument("--no-denoise", action="store_true", help="skip the denoise legs (and the records beside them)")
     ap.add_argument("--no-others", action="store_true", help="skip the C3 / C4 steps reported beside the headline")
     ap.add_argument("--serial", action="store_true",
-                    help="keep the backward's two big kernels on one stream (for per-kernel profiles)")
+                    help="launch the backward's kernels one by one (for per-kernel profiles)")
     ap.add_argument("--workload", default="c5", choices=["c3", "c4", "c5"])
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MIB",
                     help="only run a plain device copy of MIB MiB a few times (reference for the "
@@ -65,8 +87,7 @@ def main() -> int:
     import torch
 
     from opentau_amd import flash_attn_hip as fa
-    from opentau_amd.flash_attn_hip import _loader
-    from opentau_amd.workloads import make_denoise_workload, make_workload
+    from opentau_amd.workloads import make_workload
 
     if not fa.is_available():
         print(f"bench.py: HIP kernels unavailable: {fa.load_error()}", file=sys.stderr)
@@ -87,7 +108,69 @@ def main() -> int:
         print(json.dumps({"copy_bytes": n, "launches": 5}))
         return 0
 
-    w = make_workload(args.workload)
+    made = {}
+
+    def workload(name):  # (drawing a workload's tensors on the CPU takes seconds: once per name)
+        if name not in made:
+            made[name] = make_workload(name)
+        return made[name]
+
+    w = workload(args.workload)
+    rec = bench_train(torch, fa, w, dev, args.steps, args.warmup)
+    result = {
+        "metric": "block-causal attn fwd+bwd TFLOP/s on unmasked FLOPs (cosmos3 shape, 1 GPU)",
+        "value": rec["tflops"],
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": rec["ms_per_step"],
+        "ms_per_step_event_median": rec["ms_per_step_event_median"],
+        "ms_per_step_event_min": rec["ms_per_step_event_min"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{w.name}: bf16 fwd+bwd B{w.B} H{w.H} Hkv{w.Hkv} D{w.D} S{w.S} "
+                        f"({w.n_prefix} prefix in block 0, text valid {w.text_lo}..{w.text_hi}, "
+                        f"{w.n_causal} causal, {w.n_action}-token action block)",
+            "unmasked_pairs": rec["unmasked_pairs"],
+            "flops_per_step": rec["flops_per_step"],
+            "pct_of_bf16_mfma_peak": rec["pct_of_bf16_mfma_peak"],
+        },
+        "roofline": rec["roofline"],
+    }
+    del rec
+    torch.cuda.empty_cache()
+
+    if not args.no_denoise:
+        from opentau_amd.workloads import make_denoise_workload
+
+        result["denoise"] = bench_denoise(torch, fa, make_denoise_workload, dev, "c2", layers=18, steps=10)
+        if args.workload == "c5" and not args.no_others:
+            result["denoise_c4"] = bench_denoise(torch, fa, make_denoise_workload, dev, "c4", layers=34, steps=5)
+            others = {}
+            for n in ("c3", "c4"):
+                r = bench_train(torch, fa, workload(n), dev, 20, 3)
+                others[n] = {k: r[k] for k in ("workload", "ms_per_step", "ms_per_step_event_median",
+                                               "ms_per_step_event_min", "tflops", "pct_of_bf16_mfma_peak",
+                                               "roofline")}
+            result["other_workloads"] = others
+            result["dispatch"] = {n: bench_dispatch(torch, fa, workload(n), dev) for n in ("c3", "c5")}
+            result["rope"] = bench_rope(torch, dev)
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(torch, workload(args.workload))
+    print(json.dumps(result))
+    return 0
+
+
+def bench_train(torch, fa, w, dev, steps, warmup):
+    """Forward + backward steps of a training configuration through the C ABI: the timed region (wall
+    clock over ``steps`` steps, HIP events around each), then every kernel of the step alone."""
+    from opentau_amd.flash_attn_hip import _loader
+
     pairs = w.pairs()
     unit = w.D * w.H * pairs  # FLOPs per "GEMM unit" / 2
     ids = [t.to(dev) for t in w.block_ids()]
@@ -98,12 +181,12 @@ def main() -> int:
     ws_b = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
     parts = ("fwd", "bwd_delta", "bwd_dq", "bwd_dkv")
 
-    def step(ready=False):
+    def step():
         """One pass of the hot path: the forward call and the backward call, each with the pass
-        over the ids that makes its tile summaries (a model would make them once for all its
+        over the ids that makes its tile summaries (a model makes them once for all its
         layers; here every step pays for them)."""
-        _, lse = fa.forward_raw(q, k, v, *ids, w.scale, workspace=ws_f, summary_ready=ready, out=out)
-        fa.backward_raw(go, q, k, v, out, lse, *ids, w.scale, workspace=ws_b, summary_ready=ready, grads=grads)
+        _, lse = fa.forward_raw(q, k, v, *ids, w.scale, workspace=ws_f, out=out)
+        fa.backward_raw(go, q, k, v, out, lse, *ids, w.scale, workspace=ws_b, grads=grads)
         return lse
 
     def step_by_kernel(ev):
@@ -117,21 +200,25 @@ def main() -> int:
             ev[2 + n].record()
 
     step()
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
+    step_ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for s in range(args.steps):
+    for s in range(steps):
+        step_ev[s][0].record()
         step()
+        step_ev[s][1].record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    ms_per_step = (t1 - t0) * 1e3 / steps
+    ev_ms = [a.elapsed_time(b) for a, b in step_ev]
     # per-kernel durations (HIP events on the stream of the launches), outside the timed region
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(args.steps)]
-    for s in range(args.steps):
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(steps)]
+    for s in range(steps):
         step_by_kernel(events[s])
     torch.cuda.synchronize()
-    part_ms = {p: sum(e[i].elapsed_time(e[i + 1]) for e in events) / args.steps for i, p in enumerate(parts)}
+    part_ms = {p: sum(e[i].elapsed_time(e[i + 1]) for e in events) / steps for i, p in enumerate(parts)}
     tflops = 14 * unit / (ms_per_step * 1e-3) / 1e12
 
     # Unmasked FLOPs each kernel is credited with.  The backward's five products
@@ -140,85 +227,77 @@ def main() -> int:
     credit = {"fwd": 4 * unit, "bwd_delta": 0, "bwd_dq": 4 * unit, "bwd_dkv": 6 * unit}
     dom = max(("fwd", "bwd_dq", "bwd_dkv"), key=lambda p: part_ms[p])
     achieved = credit[dom] / (part_ms[dom] * 1e-3) / 1e12
+    traffic = hbm_traffic_from_profile(w.name)
     roofline = {
         "bound": "mfma",
         "kernel": {"fwd": "fwd_mfma_kernel", "bwd_dq": "bwd_dq_kernel",
-                   "bwd_dkv": "bwd_dkv_pair_kernel" if w.D == 128 else "bwd_dkv_kernel"}[dom],
+                   "bwd_dkv": "bwd_dkv_pair_kernel" if w.D == 128 else "bwd_dkv_kernel (dV launch + dK launch)"}[dom],
         "achieved": round(achieved, 2),
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-        "traffic": HBM_TRAFFIC_BYTES.get((w.name, dom)),
+        "traffic": traffic.get(dom),
+        "traffic_source": "profiles/hbm_traffic_counters.txt (counter runs of this command, not this run)"
+                          if traffic.get(dom) else None,
         "kernel_ms": {p: round(part_ms[p], 4) for p in parts},
         "kernel_tflops": {p: round(credit[p] / (part_ms[p] * 1e-3) / 1e12, 2) for p in parts if credit[p]},
+        "kernel_traffic": {p: traffic.get(p) for p in ("fwd", "bwd_dq", "bwd_dkv")},
         "step_frac": round(tflops / PEAK_BF16_TFLOPS, 4),
     }
-
-    result = {
-        "metric": "block-causal attn fwd+bwd TFLOP/s on unmasked FLOPs (cosmos3 shape, 1 GPU)",
-        "value": round(tflops, 2),
-        "unit": "TFLOP/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+    return {
+        "workload": f"{w.name}: bf16 fwd+bwd B{w.B} H{w.H} Hkv{w.Hkv} D{w.D} S{w.S}",
         "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "bf16",
-        "data": "synthetic",
-        "config": {
-            "workload": f"{w.name}: bf16 fwd+bwd B{w.B} H{w.H} Hkv{w.Hkv} D{w.D} S{w.S} "
-                        f"({w.n_prefix} prefix in block 0, text valid {w.text_lo}..{w.text_hi}, "
-                        f"{w.n_causal} causal, {w.n_action}-token action block)",
-            "unmasked_pairs": pairs,
-            "flops_per_step": 14 * unit,
-            "pct_of_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2),
-        },
+        "ms_per_step_event_median": round(statistics.median(ev_ms), 4),
+        "ms_per_step_event_min": round(min(ev_ms), 4),
+        "tflops": round(tflops, 2),
+        "pct_of_bf16_mfma_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2),
+        "unmasked_pairs": pairs,
+        "flops_per_step": 14 * unit,
         "roofline": roofline,
     }
 
-    if not args.no_denoise:
-        result["denoise"] = bench_denoise(torch, fa, make_denoise_workload, dev)
-        if args.workload == "c5" and not args.no_others:
-            result["other_workloads"] = {n: bench_step_only(torch, fa, make_workload, dev, n) for n in ("c3", "c4")}
-            result["rope"] = bench_rope(torch, dev)
-    if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(torch, make_workload, args.workload)
-    print(json.dumps(result))
-    return 0
 
+def bench_dispatch(torch, fa, w, dev, steps=20, warmup=3):
+    """What the PyTorch-facing call adds to the raw C-ABI step: the same forward + backward through
+    ``flash_attention_forward`` and autograd (outputs and gradients allocated by the framework), once
+    with a plain tuple of block ids (the traced custom ops; workspace and summaries per call) and once
+    with a ``BlockIds`` (workspace and summaries kept across calls), HIP-event median per step."""
+    from opentau_amd import attention
 
-def bench_step_only(torch, fa, make_workload, dev, name, steps=20, warmup=3):
-    """Forward + backward step of another training configuration (the head_dim 256 shapes):
-    the same measurement as the headline, without the per-kernel breakdown."""
-    w = make_workload(name)
-    ids = [t.to(dev) for t in w.block_ids()]
-    q, k, v, go = (t.to(dev) for t in (w.q, w.k, w.v, w.d_out))
-    grads = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v))
-    out = torch.empty_like(q)
+    plain = tuple(t.to(dev) for t in w.block_ids())
+    held = fa.BlockIds(*plain)
+    q, k, v = (t.to(dev).requires_grad_(True) for t in (w.q, w.k, w.v))
+    go = w.d_out.to(dev).reshape(w.B, w.S, w.H * w.D)
+    out = {}
+    for name, ids in (("autograd_op_plain_ids_ms", plain), ("autograd_block_ids_ms", held)):
+        ms = []
+        for s in range(warmup + steps):
+            q.grad = k.grad = v.grad = None
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            attention.flash_attention_forward(None, ids, w.B, w.D, q, k, v).backward(go)
+            e1.record()
+            torch.cuda.synchronize()
+            if s >= warmup:
+                ms.append(e0.elapsed_time(e1))
+        out[name] = round(statistics.median(ms), 4)
     ws_f = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
     ws_b = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
-
-    def step():
-        _, lse = fa.forward_raw(q, k, v, *ids, w.scale, workspace=ws_f, out=out)
-        fa.backward_raw(go, q, k, v, out, lse, *ids, w.scale, workspace=ws_b, grads=grads)
-
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(steps):
-        step()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / steps
-    flops = 14 * w.D * w.H * w.pairs()
-    return {
-        "workload": f"{w.name}: bf16 fwd+bwd B{w.B} H{w.H} Hkv{w.Hkv} D{w.D} S{w.S}",
-        "ms_per_step": round(ms, 4),
-        "tflops": round(flops / (ms * 1e-3) / 1e12, 2),
-        "pct_of_bf16_mfma_peak": round(100 * flops / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 2),
-    }
+    qd, kd, vd, god = q.detach(), k.detach(), v.detach(), w.d_out.to(dev)
+    grads, o = (torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)), torch.empty_like(qd)
+    ms = []
+    for s in range(warmup + steps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        _, lse = fa.forward_raw(qd, kd, vd, *plain, w.scale, workspace=ws_f, out=o)
+        fa.backward_raw(god, qd, kd, vd, o, lse, *plain, w.scale, workspace=ws_b, grads=grads)
+        e1.record()
+        torch.cuda.synchronize()
+        if s >= warmup:
+            ms.append(e0.elapsed_time(e1))
+    out["raw_c_abi_ms"] = round(statistics.median(ms), 4)
+    out["workload"] = f"{w.name}: bf16 fwd+bwd B{w.B} H{w.H} Hkv{w.Hkv} D{w.D} S{w.S}, one step at a time (synchronised)"
+    return out
 
 
 def bench_rope(torch, dev, calls=50, warmup=5):
@@ -263,16 +342,16 @@ def bench_rope(torch, dev, calls=50, warmup=5):
     return out
 
 
-def bench_denoise(torch, fa, make_denoise_workload, dev):
-    """pi0.5 inference attention: 18 prefix calls, then 10 steps x 18 cached-suffix calls."""
-    layers, steps = 18, 10
-    dw = make_denoise_workload("c2", layers=layers, steps=steps, device=dev, distinct=36)
+def bench_denoise(torch, fa, make_denoise_workload, dev, name, layers, steps):
+    """Inference attention of one ``sample_actions``: ``layers`` prefix calls, then ``steps`` x ``layers``
+    KV-cached suffix calls (pi0.5: 18, 10 x 18 at B=8; pi0.6: 34, 5 x 34 at B=16)."""
+    dw = make_denoise_workload(name, layers=layers, steps=steps, device=dev, distinct=36, distinct_prefix=6)
     w = dw.base
     npre, nact = w.n_prefix, w.n_action
     scale = w.scale
     pre_ids, suf_ids = dw.prefix_ids, dw.suffix_ids
     caches = [(kk[:, :npre], vv[:, :npre]) for (_, kk, vv) in dw.prefix]
-    ws_p = torch.empty(1 << 20, dtype=torch.uint8, device=dev)
+    ws_p = torch.empty(4 << 20, dtype=torch.uint8, device=dev)
     ws_s = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
     out_p = torch.empty_like(dw.prefix[0][0])
     out_s = torch.empty_like(dw.suffix[0][0])
@@ -281,7 +360,7 @@ def bench_denoise(torch, fa, make_denoise_workload, dev):
         if ev:
             ev[0].record()
         for li in range(layers):
-            qq, kk, vv = dw.prefix[li]
+            qq, kk, vv = dw.prefix[li % len(dw.prefix)]
             fa.forward_raw(qq, kk, vv, *pre_ids, scale, workspace=ws_p, summary_ready=li > 0, out=out_p,
                            want_lse=False)
         if ev:
@@ -290,7 +369,7 @@ def bench_denoise(torch, fa, make_denoise_workload, dev):
         for _ in range(steps):
             for li in range(layers):
                 qs, kn, vn = dw.suffix[n % len(dw.suffix)]
-                kc, vc = caches[li]
+                kc, vc = caches[li % len(caches)]
                 fa.forward_raw(qs, kc, vc, *suf_ids, scale, kn, vn, kvcache=True, workspace=ws_s,
                                summary_ready=n > 0, out=out_s, want_lse=False)
                 n += 1
@@ -307,8 +386,8 @@ def bench_denoise(torch, fa, make_denoise_workload, dev):
         run(evs[r])
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / reps
-    pre_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / reps
-    suf_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / reps
+    pre_ms = statistics.median(e[0].elapsed_time(e[1]) for e in evs)
+    suf_ms = statistics.median(e[1].elapsed_time(e[2]) for e in evs)
     valid = w.pad[:, :npre].sum().item()  # valid cached keys over the batch
     kv_bytes = 2 * (valid + w.B * nact) * w.Hkv * w.D * 2
     qo_bytes = 2 * w.B * nact * w.H * w.D * 2
@@ -318,8 +397,9 @@ def bench_denoise(torch, fa, make_denoise_workload, dev):
     gbps = bytes_call / (suf_call_us * 1e-6) / 1e9
     pairs_pre = int((w.pad[:, :npre].sum(1) ** 2).sum())
     pre_tflops = 4 * w.D * w.H * pairs_pre * layers / (pre_ms * 1e-3) / 1e12
+    suf_pairs = int((w.pad[:, :npre].sum(1) + nact).sum()) * nact
     return {
-        "workload": f"c2: pi0.5 inference bf16 B{w.B} H{w.H} Hkv{w.Hkv} D{w.D}, {layers} prefix calls "
+        "workload": f"{name}: inference bf16 B{w.B} H{w.H} Hkv{w.Hkv} D{w.D}, {layers} prefix calls "
                     f"(S{npre}) + {steps}x{layers} suffix calls (Sq{nact}, Sk{npre + nact})",
         "total_ms": round(pre_ms + suf_ms, 3),
         "wall_ms": round(wall_ms, 3),
@@ -330,20 +410,23 @@ def bench_denoise(torch, fa, make_denoise_workload, dev):
         "suffix_algorithmic_bytes_per_call": int(bytes_call),
         "suffix_GBps": round(gbps, 1),
         "suffix_hbm_frac": round(gbps / PEAK_HBM_GBPS, 4),
+        "suffix_tflops": round(4 * w.D * w.H * suf_pairs / (suf_call_us * 1e-6) / 1e12, 1),
     }
 
 
-def cpu_baseline(torch, make_workload, name, budget_s=12.0):
+def cpu_baseline(torch, w, budget_s=12.0):
     """The eager CPU oracle (reference algorithm) on a bounded part of the same workload.
 
     The workload is walked one (sample, kv head) slice at a time -- the kv head's
     K/V with the query heads of its group, forward + backward by autograd -- until
     about ``budget_s`` seconds of CPU work are done; the rate is unmasked FLOPs of
-    the slices done over the time they took.
+    the slices done over the time they took.  The tensors go in as the workload has
+    them (bf16): the eager path upcasts Q and K itself and runs P.V and its gradients
+    in the tensors' own type (``src/opentau/policies/pi05/paligemma_with_expert.py:929-947``).
     """
     from oracle import eager
 
-    w = make_workload(name)
+    name = w.name
     grp = w.H // w.Hkv
     ids = w.block_ids()
     cores = torch.get_num_threads()
@@ -353,9 +436,8 @@ def cpu_baseline(torch, make_workload, name, budget_s=12.0):
         pairs_b = int(eager.dense_mask_from_block_ids(*sl).sum())
         for hk in range(w.Hkv):
             hs = slice(hk * grp, (hk + 1) * grp)
-            # (fp32 copies: the oracle is the reference's eager arithmetic, not a bf16 CPU kernel)
-            q, go = w.q[b : b + 1, :, hs].float(), w.d_out[b : b + 1, :, hs].float()
-            k, v = w.k[b : b + 1, :, hk : hk + 1].float(), w.v[b : b + 1, :, hk : hk + 1].float()
+            q, go = w.q[b : b + 1, :, hs], w.d_out[b : b + 1, :, hs]
+            k, v = w.k[b : b + 1, :, hk : hk + 1], w.v[b : b + 1, :, hk : hk + 1]
             t0 = time.perf_counter()
             eager.eager_grads(q, k, v, go, *sl, w.scale)
             dt += time.perf_counter() - t0
@@ -370,10 +452,11 @@ def cpu_baseline(torch, make_workload, name, budget_s=12.0):
         "unit": "TFLOP/s",
         "cores": cores,
         "kind": "port",
+        "dtype": str(w.q.dtype).replace("torch.", ""),
         "seconds": round(dt, 2),
         "sample": f"{name}: first {done} of {w.B * w.Hkv} (sample, kv head) slices, each the kv head with its "
-                  f"{grp} query heads, eager fwd+bwd by autograd, {flops / 1e9:.0f} GFLOP unmasked; "
-                  f"torch CPU {cores} threads of {os.cpu_count()} cpus",
+                  f"{grp} query heads, eager fwd+bwd by autograd on the {str(w.q.dtype).replace('torch.', '')} "
+                  f"tensors, {flops / 1e9:.0f} GFLOP unmasked; torch CPU {cores} threads of {os.cpu_count()} cpus",
     }
 
 

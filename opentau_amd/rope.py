@@ -29,10 +29,15 @@ _NORM_KINDS = {"gemma3": 0, "qwen3": 1}  # enum bcattn_norm_kind
 def rope_timescale(head_dim: int, max_wavelength: float, device: torch.device) -> torch.Tensor:
     """``max_wavelength ** (2 i / head_dim)`` for the ``head_dim / 2`` bands, fp32, computed with the
     same torch ops on the same device as ``paligemma_with_expert.py:84-85`` so the kernel divides
-    by the very numbers the reference does.  Cached per (head_dim, wavelength, device)."""
+    by the very numbers the reference does.  Cached per (head_dim, wavelength, device).  The first
+    call for a key must come outside HIP-graph capture: a tensor made while a stream is capturing lives
+    in the graph's memory pool and holds data only during a replay, so it must not be kept."""
     key = (head_dim, max_wavelength, str(device))
     t = _timescales.get(key)
     if t is None:
+        if torch.device(device).type == "cuda" and torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("rope_timescale: first use of this (head_dim, wavelength, device) under graph "
+                               "capture; call the rotary embedding once before capturing")
         exponents = (2.0 / head_dim) * torch.arange(head_dim // 2, dtype=torch.float32, device=device)
         t = (max_wavelength**exponents).to(torch.float32).contiguous()
         _timescales[key] = t

@@ -144,11 +144,12 @@ class DenoiseWorkload:
 
 
 def make_denoise_workload(name: str = "c2", *, layers: int = 18, steps: int = 10, device="cpu",
-                          distinct: int | None = None) -> DenoiseWorkload:
+                          distinct: int | None = None, distinct_prefix: int | None = None) -> DenoiseWorkload:
     """Inputs of one ``sample_actions``: ``layers`` prefix calls, ``layers*steps`` suffix calls.
 
     ``distinct`` bounds how many different suffix input sets are drawn (they are
-    cycled); ``None`` draws one per (layer, step).  Prefix mask: all of block 0;
+    cycled); ``None`` draws one per (layer, step).  ``distinct_prefix`` does the same for
+    the per-layer prefix sets (``dw.prefix[i % len(dw.prefix)]`` is layer ``i``'s).  Prefix mask: all of block 0;
     suffix mask: cached columns (``INT_BLK_MIN``, validity = prefix padding) then
     one 50-token block.
     """
@@ -167,7 +168,7 @@ def make_denoise_workload(name: str = "c2", *, layers: int = 18, steps: int = 10
     def draw(s, heads):
         return torch.randn(b, s, heads, d, generator=gen).to(base.dtype).to(device)
 
-    for _ in range(layers):
+    for _ in range(layers if distinct_prefix is None else min(distinct_prefix, layers)):
         dw.prefix.append((draw(npre, h), draw(npre, hkv), draw(npre, hkv)))
     n_suf = layers * steps if distinct is None else min(distinct, layers * steps)
     for _ in range(n_suf):
