@@ -159,6 +159,7 @@ def main() -> int:
                                                "roofline")}
             result["other_workloads"] = others
             result["dispatch"] = {n: bench_dispatch(torch, fa, workload(n), dev) for n in ("c3", "c5")}
+            result["reference_harness"] = bench_reference_harness(torch, fa, dev)
             result["rope"] = bench_rope(torch, dev)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, workload(args.workload))
@@ -300,6 +301,65 @@ def bench_dispatch(torch, fa, w, dev, steps=20, warmup=3):
     return out
 
 
+def bench_reference_harness(torch, fa, dev):
+    """The shapes and the protocol of the reference's own harness
+    (``src/opentau/scripts/benchmark_flash_attn.py``: ``:405`` four H8 Hkv1 D256 shapes, forward and
+    forward + backward through the autograd op; ``:329-388`` the long-context forward sweep, B1,
+    S = 4096 ... 98 304), prefix-LM mask (first half one block, second half strictly causal,
+    ``:76-85``); 3 warm-ups, HIP events around 20 (sweep: 5) iterations (``:108-122``, ``:345-361``)."""
+
+    def ids_for(b, s):
+        att = torch.zeros(b, s, dtype=torch.int32, device=dev)
+        att[:, s // 2:] = 1
+        return fa.make_att_block_ids(torch.ones(b, s, dtype=torch.bool, device=dev), att)
+
+    def timed(fn, iters, warm=3):
+        for _ in range(warm):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters
+
+    def pairs_of(b, s):  # first half sees the first half; row i of the second half sees keys 0..i
+        half = s // 2
+        return b * (half * half + sum(range(half + 1, s + 1)))
+
+    h, hkv, d = 8, 1, 256
+    scale = d**-0.5
+    shapes = {}
+    for b, s in ((2, 512), (2, 768), (1, 1024), (1, 2048)):
+        q = torch.randn(b, s, h, d, device=dev, dtype=torch.bfloat16)
+        k, v = (torch.randn(b, s, hkv, d, device=dev, dtype=torch.bfloat16) for _ in range(2))
+        ids = ids_for(b, s)
+
+        def fwd(q=q, k=k, v=v, ids=ids):
+            fa.flash_attn_blockmask(q, k, v, *ids, scale)
+
+        def fwd_bwd(q=q, k=k, v=v, ids=ids):
+            qq, kk, vv = (t.detach().requires_grad_(True) for t in (q, k, v))
+            fa.flash_attn_blockmask(qq, kk, vv, *ids, scale).float().sum().backward()
+
+        shapes[f"B{b} S{s}"] = {"fwd_ms": round(timed(fwd, 20), 4), "fwd_bwd_ms": round(timed(fwd_bwd, 20), 4)}
+    sweep = {}
+    for s in (4096, 8192, 16384, 32768, 65536, 98304):
+        q = torch.randn(1, s, h, d, device=dev, dtype=torch.bfloat16)
+        k, v = (torch.randn(1, s, hkv, d, device=dev, dtype=torch.bfloat16) for _ in range(2))
+        ids = ids_for(1, s)
+        torch.cuda.empty_cache()
+        torch.cuda.reset_peak_memory_stats()
+        ms = timed(lambda q=q, k=k, v=v, ids=ids: fa.flash_attn_blockmask(q, k, v, *ids, scale), 5, warm=2)
+        sweep[f"S{s}"] = {"fwd_ms": round(ms, 3), "peak_GB": round(torch.cuda.max_memory_allocated() / 1e9, 3),
+                          "tflops": round(4 * d * h * pairs_of(1, s) / (ms * 1e-3) / 1e12, 1)}
+        del q, k, v
+    return {"workload": "bf16 H8 Hkv1 D256, prefix-LM mask (second half causal), through flash_attn_blockmask",
+            "shapes": shapes, "long_context_forward": sweep}
+
+
 def bench_rope(torch, dev, calls=50, warmup=5):
     """The rotary-embedding pass that feeds the attention call (queries and keys of one layer,
     in place, bf16), at the training shapes: an HBM-bound kernel, so GB/s on its algorithmic
@@ -388,6 +448,39 @@ def bench_denoise(torch, fa, make_denoise_workload, dev, name, layers, steps):
     wall_ms = (time.perf_counter() - t0) * 1e3 / reps
     pre_ms = statistics.median(e[0].elapsed_time(e[1]) for e in evs)
     suf_ms = statistics.median(e[1].elapsed_time(e[2]) for e in evs)
+    # The same suffix calls replayed from a captured HIP graph, as a serving loop would issue them
+    # (the calls allocate nothing and stay on the captured stream): what is left is kernel time and the
+    # gaps between dependent launches, without the host's part.
+    def suffix_only():
+        n = 0
+        for _ in range(steps):
+            for li in range(layers):
+                qs, kn, vn = dw.suffix[n % len(dw.suffix)]
+                kc, vc = caches[li % len(caches)]
+                fa.forward_raw(qs, kc, vc, *suf_ids, scale, kn, vn, kvcache=True, workspace=ws_s,
+                               summary_ready=True, out=out_s, want_lse=False)
+                n += 1
+
+    graph_us = None
+    try:
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            suffix_only()
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            suffix_only()
+        graph.replay()
+        g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        g0.record()
+        for _ in range(reps):
+            graph.replay()
+        g1.record()
+        torch.cuda.synchronize()
+        graph_us = g0.elapsed_time(g1) * 1e3 / (reps * layers * steps)
+    except RuntimeError as exc:  # capture unavailable: report it, keep the eager figures
+        print(f"bench.py: graph replay of the suffix calls skipped: {exc}", file=sys.stderr)
     valid = w.pad[:, :npre].sum().item()  # valid cached keys over the batch
     kv_bytes = 2 * (valid + w.B * nact) * w.Hkv * w.D * 2
     qo_bytes = 2 * w.B * nact * w.H * w.D * 2
@@ -407,6 +500,7 @@ def bench_denoise(torch, fa, make_denoise_workload, dev, name, layers, steps):
         "prefix_tflops": round(pre_tflops, 1),
         "suffix_ms": round(suf_ms, 3),
         "suffix_us_per_call": round(suf_call_us, 2),
+        "suffix_us_per_call_graph_replay": None if graph_us is None else round(graph_us, 2),
         "suffix_algorithmic_bytes_per_call": int(bytes_call),
         "suffix_GBps": round(gbps, 1),
         "suffix_hbm_frac": round(gbps / PEAK_HBM_GBPS, 4),
