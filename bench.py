@@ -399,6 +399,37 @@ def bench_rope(torch, dev, calls=50, warmup=5):
             "gbps": round(gbps, 1),
             "hbm_frac": round(gbps / PEAK_HBM_GBPS, 4),
         }
+    # pi0.6's q_norm / k_norm in front of the rotation (C4's shape): the fused forward, and the one launch
+    # that gives the gradients of q, k and both weights (three tensors' worth of traffic: dz and x in, dx out)
+    b, length, h, hkv, d = 16, 1074, 8, 4, 256
+    gen = torch.Generator(device="cpu").manual_seed(1)
+    q = torch.randn(b, length, h, d, generator=gen).to(dev, torch.bfloat16)
+    k = torch.randn(b, length, hkv, d, generator=gen).to(dev, torch.bfloat16)
+    gq, gk, qo, ko = torch.randn_like(q), torch.randn_like(k), torch.empty_like(q), torch.empty_like(k)
+    wq, wk = (torch.randn(d, generator=gen) * 0.1).to(dev), (torch.randn(d, generator=gen) * 0.1).to(dev)
+    pos = torch.arange(length, dtype=torch.int32, device=dev)[None].expand(b, length).contiguous()
+    elems = q.numel() + k.numel()
+    legs = {
+        "c4_gemma3_norm": (lambda: rope.rope_raw(q, k, pos, 1e6, q_out=qo, k_out=ko, q_norm_weight=wq, k_norm_weight=wk),
+                           2 * 2 * elems + 4 * pos.numel(), "per-head RMS norm then rope of q and k"),
+        "c4_gemma3_norm_grad": (lambda: rope.rope_norm_bwd_raw(gq, gk, q, k, pos, 1e6, q_norm_weight=wq, k_norm_weight=wk),
+                                3 * 2 * elems + 4 * pos.numel(),
+                                "gradients of q, k and both weights of the norm + rope (with the sum of the partials)"),
+    }
+    for name, (fn, nbytes, what) in legs.items():
+        for _ in range(warmup):
+            fn()
+        t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0.record()
+        for _ in range(calls):
+            fn()
+        t1.record()
+        torch.cuda.synchronize()
+        us = t0.elapsed_time(t1) * 1e3 / calls
+        gbps = nbytes / (us * 1e-6) / 1e9
+        out[name] = {"workload": f"{what}, bf16 B{b} L{length} H{h} Hkv{hkv} D{d}", "us_per_call": round(us, 2),
+                     "algorithmic_bytes": nbytes, "gbps": round(gbps, 1), "hbm_frac": round(gbps / PEAK_HBM_GBPS, 4)}
     return out
 
 

@@ -51,7 +51,7 @@
 extern "C" {
 #endif
 
-#define BCATTN_ABI_VERSION 3
+#define BCATTN_ABI_VERSION 4
 
 enum bcattn_dtype { BCATTN_F32 = 0, BCATTN_BF16 = 1, BCATTN_F16 = 2 };
 
@@ -248,6 +248,47 @@ typedef struct bcattn_rope_params {
 enum bcattn_norm_kind { BCATTN_NORM_GEMMA3 = 0, BCATTN_NORM_QWEN3 = 1 };
 
 int bcattn_rope(const bcattn_rope_params *p, void *stream);
+
+/*
+ * Gradient of bcattn_rope with norm weights: what autograd computes through q_norm / k_norm followed
+ * by the rotation (src/opentau/policies/pi06/gemma3_with_expert.py:851-861; cosmos3's expert,
+ * src/opentau/policies/cosmos3/qwen3vl_with_expert.py:85-102, :217-224), in one launch, so that the
+ * training configurations can use the fused call as well.
+ *
+ * With y = norm(x) (rounded to the element type) and z = rotate(y):  dy = the rotation of dz by minus
+ * the angle (rounded to the element type, as the gradient of a tensor of that type is); r =
+ * rsqrt(mean(x^2) + eps), xh = x * r, dyh = dy * (1 + w) [BCATTN_NORM_GEMMA3] or dy * w rounded to
+ * the element type [BCATTN_NORM_QWEN3, whose forward rounds xh before the weight multiplies it];
+ * dx = r * (dyh - xh * mean(dyh * xh)), rounded once;  dw = sum over all (batch, position, head) rows
+ * of dy * xh (BCATTN_NORM_QWEN3: xh rounded to the element type).  A tensor whose weight pointer is
+ * null went through no norm: its dx is dy.
+ *
+ * The weight gradients come as per-workgroup partial sums, dw_partial (blocks, 2, D) fp32 with
+ * blocks = bcattn_rope_norm_bwd_blocks(p): [.][0] the q weight's, [.][1] the k weight's; the caller
+ * adds them over the first axis.  Every sum inside the kernel runs in a fixed order, so with a
+ * fixed-order sum on the caller's side the gradients are bit-repeatable.  Same limits as the forward
+ * with a norm (head_dim a power of two); fp32 up to head_dim 256.
+ */
+typedef struct bcattn_rope_norm_bwd_params {
+  bcattn_tensor dq_out, dk_out; /* (B,L,H,D), (B,L,Hkv,D) in: gradients of the rotated outputs; a null pointer skips the tensor */
+  bcattn_tensor q, k;           /* same shapes, in: the forward's inputs (before the norm) */
+  bcattn_tensor dq, dk;         /* same shapes, out: the inputs' gradients (may alias dq_out / dk_out) */
+  const int32_t *positions;     /* as in bcattn_rope_params */
+  const float *timescale;
+  const void *cos, *sin;
+  const float *q_norm_weight;   /* (D) or null */
+  const float *k_norm_weight;
+  float *dw_partial;            /* (blocks, 2, D) out */
+  int32_t B, L, H, Hkv, D;
+  int32_t n_axes;
+  int32_t dtype;
+  int32_t norm_kind;
+  float norm_eps;
+} bcattn_rope_norm_bwd_params;
+
+/* Rows of dw_partial that the call writes (its number of workgroups). */
+size_t bcattn_rope_norm_bwd_blocks(const bcattn_rope_norm_bwd_params *p);
+int bcattn_rope_norm_bwd(const bcattn_rope_norm_bwd_params *p, void *stream);
 
 #ifdef __cplusplus
 }

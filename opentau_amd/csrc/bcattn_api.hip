@@ -442,4 +442,60 @@ int bcattn_rope(const bcattn_rope_params *p, void *stream) {
   return BCATTN_OK;
 }
 
+size_t bcattn_rope_norm_bwd_blocks(const bcattn_rope_norm_bwd_params *p) {
+  if (p == nullptr || p->B <= 0 || p->L <= 0) return 0;
+  return (size_t)rope_norm_bwd_blocks(p->B, p->L, p->dq_out.ptr ? p->H : 0, p->dk_out.ptr ? p->Hkv : 0, p->D, p->dtype);
+}
+
+int bcattn_rope_norm_bwd(const bcattn_rope_norm_bwd_params *p, void *stream) {
+  if (p == nullptr) return fail(BCATTN_ERR_INVALID, "null params");
+  if (p->dtype != BCATTN_F32 && !is16(p->dtype))
+    return fail(BCATTN_ERR_UNSUPPORTED, "dtype %d not supported (0 = fp32, 1 = bf16, 2 = fp16)", p->dtype);
+  const int vec = is16(p->dtype) ? 8 : 4;
+  if (p->B < 0 || p->L < 0 || p->D <= 0 || p->n_axes < 1)
+    return fail(BCATTN_ERR_INVALID, "bad shape B=%d L=%d D=%d n_axes=%d", p->B, p->L, p->D, p->n_axes);
+  if ((int64_t)p->B * p->L >= ((int64_t)1 << 31) - 64) return fail(BCATTN_ERR_UNSUPPORTED, "B*L too large");
+  if (p->D % (2 * vec) || (p->D & (p->D - 1)) || p->D / (2 * vec) > 32)
+    return fail(BCATTN_ERR_UNSUPPORTED, "the norm's gradient needs a power-of-two head_dim of %d..%d; got %d", 2 * vec,
+                64 * vec, p->D);
+  const bool tables = p->cos != nullptr || p->sin != nullptr;
+  if (tables && (p->cos == nullptr || p->sin == nullptr)) return fail(BCATTN_ERR_INVALID, "cos and sin tables come together");
+  if (!tables && (p->positions == nullptr || p->timescale == nullptr))
+    return fail(BCATTN_ERR_INVALID, "null positions / timescale pointer");
+  if (p->norm_kind != BCATTN_NORM_GEMMA3 && p->norm_kind != BCATTN_NORM_QWEN3)
+    return fail(BCATTN_ERR_INVALID, "norm_kind %d unknown", p->norm_kind);
+  if (!(p->norm_eps >= 0.f)) return fail(BCATTN_ERR_INVALID, "norm_eps must be non-negative");
+  if (p->dw_partial == nullptr) return fail(BCATTN_ERR_INVALID, "null dw_partial");
+  int rc;
+  if ((rc = check_tensor("dq_out", p->dq_out, vec, false)) || (rc = check_tensor("dk_out", p->dk_out, vec, false))) return rc;
+  const bool hq = p->dq_out.ptr != nullptr, hk = p->dk_out.ptr != nullptr;
+  if ((rc = check_tensor("dq", p->dq, vec, hq)) || (rc = check_tensor("dk", p->dk, vec, hk))) return rc;
+  if ((rc = check_tensor("q", p->q, vec, hq && p->q_norm_weight != nullptr)) ||
+      (rc = check_tensor("k", p->k, vec, hk && p->k_norm_weight != nullptr)))
+    return rc;
+  if ((hq && p->H <= 0) || (hk && p->Hkv <= 0)) return fail(BCATTN_ERR_INVALID, "bad head counts H=%d Hkv=%d", p->H, p->Hkv);
+  if ((hq ? (int64_t)p->H : 0) + (hk ? (int64_t)p->Hkv : 0) > 16384) return fail(BCATTN_ERR_UNSUPPORTED, "more than 16384 heads");
+  RopeNormBwdArgs g;
+  g.r.q = targ(p->dq_out);
+  g.r.k = targ(p->dk_out);
+  g.r.q_out = targ(p->dq);
+  g.r.k_out = targ(p->dk);
+  g.r.positions = p->positions;
+  g.r.timescale = p->timescale;
+  g.r.cos_t = p->cos;
+  g.r.sin_t = p->sin;
+  g.r.q_w = hq ? p->q_norm_weight : nullptr;
+  g.r.k_w = hk ? p->k_norm_weight : nullptr;
+  g.r.B = p->B, g.r.L = p->L, g.r.H = p->H, g.r.Hkv = p->Hkv, g.r.D = p->D, g.r.n_axes = p->n_axes;
+  g.r.inverse = 1;
+  g.r.norm_kind = p->norm_kind;
+  g.r.eps = p->norm_eps;
+  g.xq = targ(p->q);
+  g.xk = targ(p->k);
+  g.dw_partial = p->dw_partial;
+  if ((rc = launch_rope_norm_bwd(g, p->dtype, static_cast<hipStream_t>(stream))))
+    return fail(rc, "rope norm backward launch failed: %s", hipGetErrorString(hipGetLastError()));
+  return BCATTN_OK;
+}
+
 }  // extern "C"

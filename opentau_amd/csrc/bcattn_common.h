@@ -181,6 +181,17 @@ struct RopeArgs {
 };
 int launch_rope(const RopeArgs &a, int dtype, hipStream_t st);
 
+// Gradient of the rotary call with a norm in front: q, k are the gradients of the rotated outputs,
+// xq, xk the forward's inputs (before the norm), q_out, k_out receive the inputs' gradients; every
+// workgroup leaves its share of the two weight gradients in dw_partial (workgroup, {q, k}, D).
+struct RopeNormBwdArgs {
+  RopeArgs r;  // q, k = output gradients; q_out, k_out = input gradients; inverse unused
+  TensorArg xq, xk;
+  float *dw_partial;
+};
+int rope_norm_bwd_blocks(int B, int L, int H, int Hkv, int D, int dtype);
+int launch_rope_norm_bwd(const RopeNormBwdArgs &a, int dtype, hipStream_t st);
+
 // Lets a kernel use more than 64 KB of dynamic LDS.  The attribute is per device, so a
 // bit per device remembers where it is already set and launches skip the runtime call.
 template <auto Kernel>

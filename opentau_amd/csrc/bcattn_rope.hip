@@ -16,7 +16,7 @@ namespace bcattn {
 template <typename T, int V>
 struct Vec {
   T v[V];
-} __attribute__((aligned(16)));
+} __attribute__((aligned(sizeof(T) * V)));
 
 constexpr int kRopeThreads = 256;
 constexpr int kRopeUnroll = 1;  // items a thread has in flight (measured: 2 is no faster, 4 is slower; occupancy does the overlapping)
@@ -240,6 +240,224 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeArgs a, co
       *reinterpret_cast<Vec<T, V> *>(dst[u] + half) = y2;
     }
   }
+}
+
+// ---- gradient of (per-head RMS norm, then rotation) ------------------------------------------
+// Forward: y = norm(x) rounded to T, z = rotate(y).  Given dz: dy = rotate by minus the angle (rounded to
+// T, as the gradient of a tensor of type T is), then with r = rsqrt(mean(x^2) + eps), xh = x * r and
+// dyh = dy * (1 + w) [Gemma-3] or dy * w rounded to T [expert]:  dx = r * (dyh - xh * mean(dyh * xh)), and the
+// weight's gradient is the sum over all rows of dy * xh (the expert's: xh rounded to T).
+//
+// A workgroup takes kRopeThreads / LPR consecutive tokens and a run of the rows [q's heads | k's heads]: a
+// thread keeps its token and its piece of the row (c) throughout, so its sines, cosines, weights and its
+// share of the weight gradient live in registers, and it walks the run's heads (first q's, then k's: which
+// tensor is uniform) with the next head's loads in flight.  The weight gradient is then added over the
+// lanes with the same piece, the waves (through LDS) and finally the workgroups (by the caller, over
+// dw_partial), each in a fixed order: bit-repeatable.  LPR (pieces per row half) is a power of two.
+constexpr int kRopeBwdRows = 16;  // rows per workgroup at most (beyond that the rows are split over several)
+// Elements per piece, for every type: with 8 (one 16-byte load of 16-bit elements) the registers a thread
+// holds leave three waves per SIMD; with 4 there are five, which hides the memory latency better than
+// the wider loads do (measured).
+constexpr int kRopeBwdVec = 4;
+inline int rope_bwd_groups(int rows) { return (rows + kRopeBwdRows - 1) / kRopeBwdRows; }
+
+template <typename T, int V, int LPR, bool TABLES>
+__global__ __launch_bounds__(kRopeThreads) void rope_norm_bwd_kernel(const RopeNormBwdArgs g, const int ngroups) {
+  static_assert(LPR > 0 && (LPR & (LPR - 1)) == 0 && LPR <= 64, "pieces per row half: a power of two within a wave");
+  constexpr int TB = kRopeThreads / LPR;
+  const RopeArgs &a = g.r;
+  extern __shared__ __align__(16) float dw_s[];  // (waves, {q, k}, D)
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = a.D / 2;
+  const int c = tid & (LPR - 1), t = tid / LPR;
+  const int nq = a.q.ptr ? a.H : 0, rows = nq + (a.k.ptr ? a.Hkv : 0);
+  const int chunk = blockIdx.x / ngroups, group = blockIdx.x - chunk * ngroups;  // uniform
+  const int per = (rows + ngroups - 1) / ngroups;
+  const int r0 = group * per, r1 = r0 + per < rows ? r0 + per : rows;
+
+  const int64_t tok = (int64_t)chunk * TB + t;
+  const bool live = tok < (int64_t)a.B * a.L;
+  const int b = live ? (int)(tok / a.L) : 0, l = live ? (int)(tok - (int64_t)b * a.L) : 0;
+
+  // this thread's sines and cosines: computed here (fp32), or the tables' two pieces kept as loaded
+  float sp[V], cp[V];
+  Vec<T, V> c1 = {}, c2 = {}, s1 = {}, s2 = {};
+  if constexpr (TABLES) {
+    const T *ct = reinterpret_cast<const T *>(a.cos_t) + ((int64_t)b * a.L + l) * a.D + c * V;
+    const T *st = reinterpret_cast<const T *>(a.sin_t) + ((int64_t)b * a.L + l) * a.D + c * V;
+    c1 = *reinterpret_cast<const Vec<T, V> *>(ct), c2 = *reinterpret_cast<const Vec<T, V> *>(ct + half);
+    s1 = *reinterpret_cast<const Vec<T, V> *>(st), s2 = *reinterpret_cast<const Vec<T, V> *>(st + half);
+  } else {
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const int band = c * V + e;
+      const int axis = a.n_axes > 1 ? band % a.n_axes : 0;
+      const float pos = (float)a.positions[((int64_t)axis * a.B + b) * a.L + l];
+      rope_sincos(__fdiv_rn(pos, a.timescale[band]), sp[e], cp[e]);
+    }
+  }
+  const bool gem = a.norm_kind == BCATTN_NORM_GEMMA3;
+  auto rt = [](float x) __attribute__((always_inline)) { return (float)(T)x; };
+  struct Row {
+    Vec<T, V> g1, g2, x1, x2;
+  };
+
+  // heads [h0, h1) of one tensor: gt the output's gradient, xt the forward's input, ot the input's gradient;
+  // w null: this tensor went through no norm, its gradient is dy
+  auto segment = [&](const TensorArg &gt, const TensorArg &xt, const TensorArg &ot, const float *w, const int h0,
+                     const int h1, float *out_s) __attribute__((always_inline)) {
+    const T *gsrc = reinterpret_cast<const T *>(gt.ptr) + b * gt.sb + (int64_t)l * gt.ss + c * V;
+    const T *xsrc = reinterpret_cast<const T *>(xt.ptr) + b * xt.sb + (int64_t)l * xt.ss + c * V;
+    T *dst = reinterpret_cast<T *>(const_cast<void *>(ot.ptr)) + b * ot.sb + (int64_t)l * ot.ss + c * V;
+    float w1[V], w2[V], dw[2][V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const float u1 = w ? w[c * V + e] : 0.f, u2 = w ? w[c * V + half + e] : 0.f;
+      w1[e] = gem ? 1.0f + u1 : u1;
+      w2[e] = gem ? 1.0f + u2 : u2;
+      dw[0][e] = dw[1][e] = 0.f;
+    }
+    auto load = [&](int h) __attribute__((always_inline)) {
+      Row r = {};
+      if (live && h < h1) {
+        r.g1 = *reinterpret_cast<const Vec<T, V> *>(gsrc + h * gt.sh);
+        r.g2 = *reinterpret_cast<const Vec<T, V> *>(gsrc + h * gt.sh + half);
+        if (w != nullptr) {
+          r.x1 = *reinterpret_cast<const Vec<T, V> *>(xsrc + h * xt.sh);
+          r.x2 = *reinterpret_cast<const Vec<T, V> *>(xsrc + h * xt.sh + half);
+        }
+      }
+      return r;
+    };
+    Row next = load(h0);
+    for (int h = h0; h < h1; ++h) {
+#pragma clang fp contract(off)
+      const Row cur = next;
+      next = load(h + 1);
+      float y1[V], y2[V];  // dy: the rotation by minus the angle, rounded to T
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const float g1 = (float)cur.g1.v[e], g2 = (float)cur.g2.v[e];
+        if constexpr (TABLES) {
+          y1[e] = rt(rt(g1 * (float)c1.v[e]) + rt(g2 * (float)s2.v[e]));
+          y2[e] = rt(rt(g2 * (float)c2.v[e]) + rt(-g1 * (float)s1.v[e]));
+        } else {
+          y1[e] = rt(g1 * cp[e] + g2 * sp[e]);
+          y2[e] = rt(g2 * cp[e] - g1 * sp[e]);
+        }
+      }
+      Vec<T, V> d1, d2;
+      if (w == nullptr) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) d1.v[e] = (T)y1[e], d2.v[e] = (T)y2[e];
+      } else {
+        // The expert's norm rounds xh to T before the weight multiplies it, so the gradient that reaches
+        // xh (dy * w) is rounded to T and the weight's gradient sees the rounded xh; Gemma-3's norm works
+        // in fp32 up to its result.  The row sums of x^2 and of dyh * x (r comes out of the second as a
+        // factor) go across the row's lanes side by side (neighbours, aligned to LPR).
+        float ss = 0.f, dot = 0.f, u1[V], u2[V];  // u: dyh
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          const float x1 = (float)cur.x1.v[e], x2 = (float)cur.x2.v[e];
+          ss += x1 * x1 + x2 * x2;
+          u1[e] = gem ? y1[e] * w1[e] : rt(y1[e] * w1[e]);
+          u2[e] = gem ? y2[e] * w2[e] : rt(y2[e] * w2[e]);
+          dot += u1[e] * x1 + u2[e] * x2;
+        }
+#pragma unroll
+        for (int o2 = 1; o2 < LPR; o2 <<= 1) ss += __shfl_xor(ss, o2, 64), dot += __shfl_xor(dot, o2, 64);
+        const float r = 1.0f / sqrtf(ss / (float)a.D + a.eps);
+        const float mean = r * dot / (float)a.D;  // mean(dyh * xh)
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          const float hh1 = (float)cur.x1.v[e] * r, hh2 = (float)cur.x2.v[e] * r;
+          d1.v[e] = (T)(r * (u1[e] - hh1 * mean));
+          d2.v[e] = (T)(r * (u2[e] - hh2 * mean));
+          dw[0][e] += y1[e] * (gem ? hh1 : rt(hh1));  // (threads past the last token: zeros)
+          dw[1][e] += y2[e] * (gem ? hh2 : rt(hh2));
+        }
+      }
+      if (live) {
+        *reinterpret_cast<Vec<T, V> *>(dst + h * ot.sh) = d1;
+        *reinterpret_cast<Vec<T, V> *>(dst + h * ot.sh + half) = d2;
+      }
+    }
+    if (w != nullptr) {  // lanes with the same piece -> one lane per piece and wave
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          float v = dw[j][e];
+#pragma unroll
+          for (int o2 = LPR; o2 < 64; o2 <<= 1) v += __shfl_xor(v, o2, 64);
+          if (lane < LPR) out_s[j * half + c * V + e] = v;
+        }
+    }
+  };
+  const bool has_q = r0 < nq, has_k = r1 > nq;
+  if (has_q) segment(a.q, g.xq, a.q_out, a.q_w, r0, r1 < nq ? r1 : nq, dw_s + (wave * 2 + 0) * a.D);
+  if (has_k) segment(a.k, g.xk, a.k_out, a.k_w, (r0 > nq ? r0 : nq) - nq, r1 - nq, dw_s + (wave * 2 + 1) * a.D);
+  __syncthreads();
+  // waves -> this workgroup's row of partial sums, in a fixed order
+  for (int x = tid; x < 2 * a.D; x += kRopeThreads) {
+    const bool used = x < a.D ? (has_q && a.q_w != nullptr) : (has_k && a.k_w != nullptr);
+    float v = 0.f;
+    if (used) {
+#pragma unroll
+      for (int wv = 0; wv < kRopeThreads / 64; ++wv) v += dw_s[wv * 2 * a.D + x];
+    }
+    g.dw_partial[(int64_t)blockIdx.x * 2 * a.D + x] = v;
+  }
+}
+
+template <int V>
+static int rope_norm_bwd_grid(int64_t ntok, int rows, int D) {
+  const int lpr = D / (2 * V);
+  if (lpr < 1 || lpr > 64 || rows < 1) return 0;
+  const int TB = kRopeThreads / lpr;
+  return (int)((ntok + TB - 1) / TB) * rope_bwd_groups(rows);
+}
+
+int rope_norm_bwd_blocks(int B, int L, int H, int Hkv, int D, int dtype) {
+  (void)dtype;
+  if (H + Hkv <= 0 || D <= 0) return 0;
+  return rope_norm_bwd_grid<kRopeBwdVec>((int64_t)B * L, H + Hkv, D);
+}
+
+template <typename T, int V>
+static int launch_rope_norm_bwd_t(const RopeNormBwdArgs &g, int nq, int nk, hipStream_t st) {
+  const RopeArgs &a = g.r;
+  const int lpr = a.D / (2 * V);
+  const dim3 grid((unsigned)rope_norm_bwd_grid<V>((int64_t)a.B * a.L, nq + nk, a.D)), block(kRopeThreads);
+  const int ngroups = rope_bwd_groups(nq + nk);
+  const bool tables = a.cos_t != nullptr;
+  const size_t lds = (size_t)(kRopeThreads / 64) * 2 * a.D * sizeof(float);
+#define BCATTN_ROPE_BWD_LAUNCH(LPR_)                                                          \
+  if (tables)                                                                                 \
+    hipLaunchKernelGGL((rope_norm_bwd_kernel<T, V, LPR_, true>), grid, block, lds, st, g, ngroups);    \
+  else                                                                                        \
+    hipLaunchKernelGGL((rope_norm_bwd_kernel<T, V, LPR_, false>), grid, block, lds, st, g, ngroups)
+  switch (lpr) {
+    case 1: BCATTN_ROPE_BWD_LAUNCH(1); break;
+    case 2: BCATTN_ROPE_BWD_LAUNCH(2); break;
+    case 4: BCATTN_ROPE_BWD_LAUNCH(4); break;
+    case 8: BCATTN_ROPE_BWD_LAUNCH(8); break;
+    case 16: BCATTN_ROPE_BWD_LAUNCH(16); break;
+    case 32: BCATTN_ROPE_BWD_LAUNCH(32); break;
+    case 64: BCATTN_ROPE_BWD_LAUNCH(64); break;
+    default: return BCATTN_ERR_UNSUPPORTED;
+  }
+#undef BCATTN_ROPE_BWD_LAUNCH
+  return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
+}
+
+int launch_rope_norm_bwd(const RopeNormBwdArgs &g, int dtype, hipStream_t st) {
+  const RopeArgs &a = g.r;
+  const int nq = a.q.ptr ? a.H : 0, nk = a.k.ptr ? a.Hkv : 0;
+  if ((int64_t)a.B * a.L == 0 || nq + nk == 0) return BCATTN_OK;
+  if (dtype == BCATTN_F32) return launch_rope_norm_bwd_t<float, kRopeBwdVec>(g, nq, nk, st);
+  if (dtype == BCATTN_BF16) return launch_rope_norm_bwd_t<__bf16, kRopeBwdVec>(g, nq, nk, st);
+  return launch_rope_norm_bwd_t<_Float16, kRopeBwdVec>(g, nq, nk, st);
 }
 
 template <typename T, int V>

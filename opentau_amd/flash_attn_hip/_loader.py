@@ -17,7 +17,7 @@ from pathlib import Path
 
 CSRC = Path(__file__).resolve().parent.parent / "csrc"
 LIB_PATH = CSRC / "libbcattn.so"
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 # status codes of include/bcattn.h
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_WORKSPACE, ERR_LAUNCH = 0, -1, -2, -3, -4
@@ -36,6 +36,8 @@ EXPORTS = (
     "bcattn_fwd_kvcache_static",
     "bcattn_bwd",
     "bcattn_rope",
+    "bcattn_rope_norm_bwd_blocks",
+    "bcattn_rope_norm_bwd",
 )
 
 
@@ -140,6 +142,35 @@ class RopeParams(ctypes.Structure):
     ]
 
 
+class RopeNormBwdParams(ctypes.Structure):
+    """``bcattn_rope_norm_bwd_params``."""
+
+    _fields_ = [
+        ("dq_out", Tensor4),
+        ("dk_out", Tensor4),
+        ("q", Tensor4),
+        ("k", Tensor4),
+        ("dq", Tensor4),
+        ("dk", Tensor4),
+        ("positions", ctypes.c_void_p),
+        ("timescale", ctypes.c_void_p),
+        ("cos", ctypes.c_void_p),
+        ("sin", ctypes.c_void_p),
+        ("q_norm_weight", ctypes.c_void_p),
+        ("k_norm_weight", ctypes.c_void_p),
+        ("dw_partial", ctypes.c_void_p),
+        ("B", ctypes.c_int32),
+        ("L", ctypes.c_int32),
+        ("H", ctypes.c_int32),
+        ("Hkv", ctypes.c_int32),
+        ("D", ctypes.c_int32),
+        ("n_axes", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("norm_kind", ctypes.c_int32),
+        ("norm_eps", ctypes.c_float),
+    ]
+
+
 _lock = threading.Lock()
 _lib = None
 _load_attempted = False
@@ -159,9 +190,11 @@ def _bind(lib: ctypes.CDLL) -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = ctypes.c_size_t
         fn.argtypes = [ctypes.POINTER(st)]
+    lib.bcattn_rope_norm_bwd_blocks.restype = ctypes.c_size_t
+    lib.bcattn_rope_norm_bwd_blocks.argtypes = [ctypes.POINTER(RopeNormBwdParams)]
     for name, st in (("bcattn_fwd", FwdParams), ("bcattn_fwd_kvcache", FwdParams),
                      ("bcattn_fwd_kvcache_static", FwdParams), ("bcattn_bwd", BwdParams),
-                     ("bcattn_rope", RopeParams)):
+                     ("bcattn_rope", RopeParams), ("bcattn_rope_norm_bwd", RopeNormBwdParams)):
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(st), ctypes.c_void_p]

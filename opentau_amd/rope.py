@@ -148,6 +148,74 @@ def rope_raw(
     return (q_out if q is not None else None), (k_out if k is not None else None)
 
 
+def rope_norm_bwd_raw(
+    grad_q: torch.Tensor | None,
+    grad_k: torch.Tensor | None,
+    q: torch.Tensor | None,
+    k: torch.Tensor | None,
+    positions: torch.Tensor | None,
+    max_wavelength: float = 10_000,
+    *,
+    q_norm_weight: torch.Tensor | None = None,
+    k_norm_weight: torch.Tensor | None = None,
+    norm_eps: float = 1e-6,
+    norm_kind: str = "gemma3",
+    cos: torch.Tensor | None = None,
+    sin: torch.Tensor | None = None,
+    stacked: bool = False,
+):
+    """One call of ``bcattn_rope_norm_bwd``: the gradient of :func:`rope_raw` with norm weights.
+
+    ``grad_q`` / ``grad_k``: gradients of the rotated outputs, ``q`` / ``k``: the forward's inputs, all
+    ``(B, L, H, D)`` views.  Returns ``(dq, dk, dw_q, dw_k)``; the weight gradients are fp32 ``(D,)``
+    (``None`` where there is no weight), the sum of the kernel's per-workgroup partial sums; with ``stacked``
+    they come as one ``(2, D)`` tensor instead (a row of zeros where there is no weight).
+    """
+    lib = _loader.require_library()
+    x = grad_q if grad_q is not None else grad_k
+    if x is None:
+        raise RuntimeError("rope_norm_bwd needs grad_q or grad_k")
+    code, vec = _DTYPES[x.dtype]
+    grad_q, grad_k = _strided(grad_q, vec, "grad_q"), _strided(grad_k, vec, "grad_k")
+    q, k = _strided(q, vec, "q"), _strided(k, vec, "k")
+    b, length, d = x.shape[0], x.shape[1], x.shape[3]
+    tables = cos is not None or sin is not None
+    if tables:
+        cos, sin = (t.to(device=x.device, dtype=x.dtype).contiguous() for t in (cos, sin))
+        pos, n_axes = None, 1
+    else:
+        pos, n_axes = _positions(positions, b, length)
+    # (the gradients take their operands' strides: head-major views give head-major results)
+    dq = torch.empty_like(grad_q) if grad_q is not None else None
+    dk = torch.empty_like(grad_k) if grad_k is not None else None
+    weights = []
+    for t, w in ((grad_q, q_norm_weight), (grad_k, k_norm_weight)):
+        weights.append(w.detach().to(device=x.device, dtype=torch.float32).contiguous()
+                       if (w is not None and t is not None) else None)
+    ts = None if tables else rope_timescale(d, max_wavelength, x.device)
+    p = _loader.RopeNormBwdParams()
+    p.dq_out, p.dk_out, p.q, p.k, p.dq, p.dk = _t4(grad_q), _t4(grad_k), _t4(q), _t4(k), _t4(dq), _t4(dk)
+    if tables:
+        p.cos, p.sin = cos.data_ptr(), sin.data_ptr()
+    else:
+        p.positions, p.timescale = pos.data_ptr(), ts.data_ptr()
+    p.q_norm_weight = weights[0].data_ptr() if weights[0] is not None else None
+    p.k_norm_weight = weights[1].data_ptr() if weights[1] is not None else None
+    p.B, p.L, p.D = b, length, d
+    p.H = grad_q.shape[2] if grad_q is not None else 0
+    p.Hkv = grad_k.shape[2] if grad_k is not None else 0
+    p.n_axes, p.dtype, p.norm_kind, p.norm_eps = n_axes, code, _NORM_KINDS[norm_kind], float(norm_eps)
+    blocks = int(lib.bcattn_rope_norm_bwd_blocks(ctypes.byref(p)))
+    partial = torch.empty((max(blocks, 1), 2, d), dtype=torch.float32, device=x.device)
+    p.dw_partial = partial.data_ptr()
+    with torch.cuda.device(x.device):
+        _check(lib.bcattn_rope_norm_bwd(ctypes.byref(p), _stream(x.device)), lib)
+    dw = partial[:blocks].sum(0)  # (2, D): one fixed-order reduction for both weights
+    if stacked:
+        return dq, dk, dw
+    return dq, dk, (dw[0] if weights[0] is not None else None), (dw[1] if weights[1] is not None else None)
+
+
 # The differentiable / traceable forms are torch.library ops (like the attention calls), so that
 # ``torch.compile`` traces through them with the fake implementations and autograd sees the
 # registered backward.  The rotation is orthogonal: its gradient is the rotation by minus the angle.
@@ -217,6 +285,67 @@ def _rope_tables_backward(ctx, grad_q, grad_k):
 _op_rope_tables.register_autograd(_rope_tables_backward, setup_context=_rope_tables_setup)
 
 
+# The forms with a per-head norm in front (q_norm / k_norm then the rotation): forward and gradient are
+# one launch each.  layout 0: (B, L, H, D) operands, angles from positions, Gemma-3's norm
+# (pi06/gemma3_with_expert.py:851-861); layout 1: (B, H, S, D) operands, cos / sin tables, the expert's
+# norm (cosmos3/qwen3vl_with_expert.py:217-224).
+def _norm_call(layout: int):
+    return ((lambda t: t), "gemma3") if layout == 0 else ((lambda t: t.transpose(1, 2)), "qwen3")
+
+
+@torch.library.custom_op("bcattn::rope_norm_qk", mutates_args=())
+def _op_rope_norm_qk(q: torch.Tensor, k: torch.Tensor, angles_a: torch.Tensor, angles_b: torch.Tensor,
+                     q_w: torch.Tensor, k_w: torch.Tensor, max_wavelength: float, eps: float,
+                     layout: int) -> tuple[torch.Tensor, torch.Tensor]:
+    view, kind = _norm_call(layout)
+    qo, ko = torch.empty_like(q), torch.empty_like(k)
+    kw = {"cos": angles_a, "sin": angles_b} if layout == 1 else {}
+    rope_raw(view(q), view(k), None if layout == 1 else angles_a, max_wavelength, q_out=view(qo), k_out=view(ko),
+             q_norm_weight=q_w, k_norm_weight=k_w, norm_eps=eps, norm_kind=kind, **kw)
+    return qo, ko
+
+
+@_op_rope_norm_qk.register_fake
+def _(q, k, angles_a, angles_b, q_w, k_w, max_wavelength, eps, layout):
+    return torch.empty_like(q), torch.empty_like(k)
+
+
+@torch.library.custom_op("bcattn::rope_norm_qk_bwd", mutates_args=())
+def _op_rope_norm_qk_bwd(grad_q: torch.Tensor, grad_k: torch.Tensor, q: torch.Tensor, k: torch.Tensor,
+                         angles_a: torch.Tensor, angles_b: torch.Tensor, q_w: torch.Tensor, k_w: torch.Tensor,
+                         max_wavelength: float, eps: float,
+                         layout: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    view, kind = _norm_call(layout)
+    kw = {"cos": angles_a, "sin": angles_b} if layout == 1 else {}
+    dq, dk, dw = rope_norm_bwd_raw(view(grad_q), view(grad_k), view(q), view(k), None if layout == 1 else angles_a,
+                                   max_wavelength, q_norm_weight=q_w, k_norm_weight=k_w, norm_eps=eps, norm_kind=kind,
+                                   stacked=True, **kw)
+    if layout == 1:  # (B, S, H, D) results of head-major operands: hand back head-major tensors
+        dq, dk = view(dq).contiguous(), view(dk).contiguous()
+    return dq, dk, dw
+
+
+@_op_rope_norm_qk_bwd.register_fake
+def _(grad_q, grad_k, q, k, angles_a, angles_b, q_w, k_w, max_wavelength, eps, layout):
+    return torch.empty_like(q), torch.empty_like(k), q_w.new_empty((2, q.shape[-1]), dtype=torch.float32)
+
+
+def _rope_norm_setup(ctx, inputs, output):
+    q, k, angles_a, angles_b, q_w, k_w, max_wavelength, eps, layout = inputs
+    ctx.save_for_backward(q, k, angles_a, angles_b, q_w, k_w)
+    ctx.consts = (max_wavelength, eps, layout)
+
+
+def _rope_norm_backward(ctx, grad_q, grad_k):
+    q, k, angles_a, angles_b, q_w, k_w = ctx.saved_tensors
+    dq, dk, dw = _op_rope_norm_qk_bwd(grad_q.contiguous(), grad_k.contiguous(), q, k, angles_a, angles_b,
+                                      q_w, k_w, *ctx.consts)
+    return dq, dk, None, None, dw[0].to(q_w.dtype), dw[1].to(k_w.dtype), None, None, None
+
+
+_op_rope_norm_qk.register_autograd(_rope_norm_backward, setup_context=_rope_norm_setup)
+
+
 def _rope_tables_bhsd(q, k, cos, sin, *, inverse=False, q_norm_weight=None, k_norm_weight=None, norm_eps=1e-6):
     """``q (B, H, S, D)``, ``k (B, Hkv, S, D)`` -> rotated tensors of the same shape (new storage)."""
     qo = torch.empty(q.shape, dtype=q.dtype, device=q.device)
@@ -259,14 +388,19 @@ def apply_rope_qk(
 
     With norm weights: ``apply_rope(q_norm(q), ...)`` and ``apply_rope(k_norm(k), ...)`` of
     ``src/opentau/policies/pi06/gemma3_with_expert.py:851-861`` where the norms are Gemma-3's
-    (``x * rsqrt(mean(x^2) + eps) * (1 + weight)``, rounded to ``x.dtype``); that form is
-    inference-only.  ``q_out`` / ``k_out`` may be the inputs themselves (in place) or views of
+    (``x * rsqrt(mean(x^2) + eps) * (1 + weight)``, rounded to ``x.dtype``); differentiable in ``q``,
+    ``k`` and both weights (one more launch for all four gradients).  ``q_out`` / ``k_out`` may be the inputs themselves (in place) or views of
     other storage, e.g. ``cache_k[:, n0:n0 + L]`` of a preallocated key cache.
     """
     norm = q_norm_weight is not None or k_norm_weight is not None
-    if _needs_graph(q, k):
-        if norm or q_out is not None or k_out is not None:
-            raise RuntimeError("apply_rope_qk is differentiable / traceable only without norm weights and output arguments")
+    if _needs_graph(q, k, *(w for w in (q_norm_weight, k_norm_weight) if w is not None)):
+        if q_out is not None or k_out is not None:
+            raise RuntimeError("apply_rope_qk is differentiable / traceable only without output arguments")
+        if norm:
+            if q_norm_weight is None or k_norm_weight is None:
+                raise RuntimeError("the differentiable form takes both norm weights (or neither)")
+            return _op_rope_norm_qk(q, k, positions, positions, q_norm_weight, k_norm_weight, float(max_wavelength),
+                                    float(norm_eps), 0)
         return _op_rope_qk(q, k, positions, float(max_wavelength), False)
     return rope_raw(q, k, positions, max_wavelength, q_out=q_out, k_out=k_out, q_norm_weight=q_norm_weight,
                     k_norm_weight=k_norm_weight, norm_eps=norm_eps)
@@ -290,18 +424,21 @@ def apply_rotary_pos_emb(
     ``cos`` / ``sin`` are ``(B, S, D)`` in the tensors' dtype, ``q`` / ``k`` are ``(B, H, S, D)`` with
     ``unsqueeze_dim=1`` (the expert's layout) or ``(B, S, H, D)`` with ``unsqueeze_dim=2``; every product
     and sum is rounded to that dtype.  Differentiable in ``q`` and ``k``.  With norm weights the expert's
-    per-head RMS norm (``ExpertRMSNorm``, ``:85-102``) runs in front, i.e. ``:217-224`` in one call
-    (inference only).
+    per-head RMS norm (``ExpertRMSNorm``, ``:85-102``) runs in front, i.e. ``:217-224`` in one call,
+    differentiable in ``q``, ``k`` and the weights.
     """
     if unsqueeze_dim not in (1, 2):
         raise RuntimeError("unsqueeze_dim must be 1 (B, H, S, D) or 2 (B, S, H, D)")
     if unsqueeze_dim == 2:
         q, k = q.transpose(1, 2), k.transpose(1, 2)
     norm = q_norm_weight is not None or k_norm_weight is not None
-    if _needs_graph(q, k):
+    if _needs_graph(q, k, *(w for w in (q_norm_weight, k_norm_weight) if w is not None)):
         if norm:
-            raise RuntimeError("apply_rotary_pos_emb is differentiable / traceable only without norm weights")
-        qo, ko = _op_rope_tables(q, k, cos, sin, False)
+            if q_norm_weight is None or k_norm_weight is None:
+                raise RuntimeError("the differentiable form takes both norm weights (or neither)")
+            qo, ko = _op_rope_norm_qk(q, k, cos, sin, q_norm_weight, k_norm_weight, 0.0, float(norm_eps), 1)
+        else:
+            qo, ko = _op_rope_tables(q, k, cos, sin, False)
     else:
         qo, ko = _rope_tables_bhsd(q, k, cos, sin, q_norm_weight=q_norm_weight, k_norm_weight=k_norm_weight,
                                    norm_eps=norm_eps)

@@ -121,3 +121,19 @@ def rope_tables(positions: torch.Tensor, head_dim: int, max_wavelength: float = 
     freqs = positions.to(torch.float32).unsqueeze(-1) / timescale
     emb = torch.cat([freqs, freqs], dim=-1)
     return emb.cos().to(dtype), emb.sin().to(dtype)
+
+
+def norm_rope_backward(x, weight, grad_out, *, kind, positions=None, max_wavelength: float = 10_000, cos=None,
+                       sin=None, eps: float = 1e-6):
+    """``(dx, dweight)`` of the per-head norm followed by the rotation, by autograd through the functions
+    above.  ``kind`` ``"gemma3"``: ``x (B, L, H, D)``, ``apply_rope(gemma3_rms_norm(x))`` with ``positions``
+    (``pi06/gemma3_with_expert.py:851-861``); ``"qwen3"``: ``x (B, H, S, D)``, the expert's norm then
+    ``apply_rotary_pos_emb`` with ``cos`` / ``sin`` (``cosmos3/qwen3vl_with_expert.py:217-224``)."""
+    x = x.detach().clone().requires_grad_(True)
+    weight = weight.detach().clone().requires_grad_(True)
+    if kind == "gemma3":
+        out = apply_rope(gemma3_rms_norm(x, weight, eps), positions, max_wavelength)
+    else:
+        out = apply_rotary_pos_emb(expert_rms_norm(x, weight, eps), x[:, :0], cos, sin)[0]
+    out.backward(grad_out)
+    return x.grad, weight.grad

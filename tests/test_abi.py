@@ -39,6 +39,7 @@ def test_struct_layout_matches_header(tmp_path):
         "bcattn_fwd_params": (_loader.FwdParams, [f[0] for f in _loader.FwdParams._fields_]),
         "bcattn_bwd_params": (_loader.BwdParams, [f[0] for f in _loader.BwdParams._fields_]),
         "bcattn_rope_params": (_loader.RopeParams, [f[0] for f in _loader.RopeParams._fields_]),
+        "bcattn_rope_norm_bwd_params": (_loader.RopeNormBwdParams, [f[0] for f in _loader.RopeNormBwdParams._fields_]),
     }
     lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "bcattn.h"', "int main(void) {"]
     for cname, (_, names) in fields.items():

@@ -243,6 +243,127 @@ def test_expert_norm_then_rotary_tables(dtype):
             assert rel_l2(a.float(), e.float()) <= 2e-3 and float((a != e).float().mean()) <= 2e-2, name
 
 
+def _close_grad(got, want, dtype, what):
+    """Gradients of a 16-bit tensor: rel-L2 <= 1e-2 and max-abs within two rounding steps of the largest
+    expected element (a gradient's scale is the workload's, not 1); fp32: rel-L2 <= 1e-5."""
+    r = rel_l2(got.float(), want.float())
+    if dtype == torch.float32:
+        assert r <= 1e-5, f"{what}: rel-L2 {r:.3e}"
+    else:
+        step = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+        lim = max(2e-2, 2 * step * float(want.float().abs().max()))
+        assert r <= 1e-2 and max_abs(got.float(), want.float()) <= lim, f"{what}: rel-L2 {r:.3e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("b,length,h,hkv,d,axes", [
+    (2, 40, 8, 4, 256, 0),    # pi0.6's backbone heads
+    (1, 131, 4, 1, 128, 3),   # MRoPE positions, a token count that is no multiple of a workgroup's share
+    (3, 5, 2, 2, 32, 0),
+    (2, 300, 8, 1, 256, 0),   # several workgroups' partial weight gradients
+])
+def test_fused_gemma3_norm_rope_gradients(dtype, b, length, h, hkv, d, axes):
+    """Gradients of q_norm / k_norm then apply_rope (pi06/gemma3_with_expert.py:851-861) w.r.t. q, k and both
+    weights from one launch, against autograd through the oracle's norm and rotation."""
+    q, k = g(randn((b, length, h, d), dtype, 1) * 3.0), g(randn((b, length, hkv, d), dtype, 2) * 0.2)
+    wq, wk = g(randn((d,), torch.float32, 3) * 0.3), g(randn((d,), torch.float32, 4) * 0.3)
+    gq, gk = g(randn((b, length, h, d), dtype, 5)), g(randn((b, length, hkv, d), dtype, 6))
+    pos = g(positions(b, length, 7, axes=axes))
+
+    def run():
+        leaves = [t.clone().requires_grad_(True) for t in (q, k, wq, wk)]
+        qo, ko = hip_rope.apply_rope_qk(leaves[0], leaves[1], pos, 1_000_000, q_norm_weight=leaves[2],
+                                        k_norm_weight=leaves[3], norm_eps=1e-6)
+        torch.autograd.backward([qo, ko], [gq, gk])
+        return [qo.detach(), ko.detach()] + [t.grad for t in leaves]
+
+    got = run()
+    plain = hip_rope.apply_rope_qk(q, k, pos, 1_000_000, q_norm_weight=wq, k_norm_weight=wk, norm_eps=1e-6)
+    assert torch.equal(got[0], plain[0]) and torch.equal(got[1], plain[1])  # the same forward kernel
+    want_q = oracle.norm_rope_backward(q, wq, gq, kind="gemma3", positions=pos, max_wavelength=1_000_000)
+    want_k = oracle.norm_rope_backward(k, wk, gk, kind="gemma3", positions=pos, max_wavelength=1_000_000)
+    _close_grad(got[2], want_q[0], dtype, "dq")
+    _close_grad(got[3], want_k[0], dtype, "dk")
+    assert got[4].dtype == torch.float32 and got[4].shape == (d,)
+    # the weight gradients are sums over b * length * heads rows, kept in fp32 on both sides
+    for a, e, name in ((got[4], want_q[1], "dwq"), (got[5], want_k[1], "dwk")):
+        r = rel_l2(a, e)
+        assert r <= (1e-5 if dtype == torch.float32 else 2e-3), f"{name}: rel-L2 {r:.3e}"
+    again = run()
+    for a, e in zip(again, got):  # fixed summation order: bit-repeatable
+        assert torch.equal(a, e)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_gemma3_norm_gradients_with_weights_in_the_element_type(dtype):
+    """Weights stored in the tensors' type (a model cast to bf16): the weight gradient comes back in it."""
+    b, length, h, hkv, d = 2, 33, 4, 2, 128
+    q, k = g(randn((b, length, h, d), dtype, 1)), g(randn((b, length, hkv, d), dtype, 2))
+    wq, wk = g(randn((d,), torch.float32, 3) * 0.3).to(dtype), g(randn((d,), torch.float32, 4) * 0.3).to(dtype)
+    gq, gk = g(randn((b, length, h, d), dtype, 5)), g(randn((b, length, hkv, d), dtype, 6))
+    pos = g(positions(b, length, 7))
+    leaves = [t.clone().requires_grad_(True) for t in (q, k, wq, wk)]
+    qo, ko = hip_rope.apply_rope_qk(leaves[0], leaves[1], pos, q_norm_weight=leaves[2], k_norm_weight=leaves[3])
+    torch.autograd.backward([qo, ko], [gq, gk])
+    want_q = oracle.norm_rope_backward(q, wq, gq, kind="gemma3", positions=pos)
+    want_k = oracle.norm_rope_backward(k, wk, gk, kind="gemma3", positions=pos)
+    assert leaves[2].grad.dtype == dtype
+    _close_grad(leaves[0].grad, want_q[0], dtype, "dq")
+    _close_grad(leaves[1].grad, want_k[0], dtype, "dk")
+    _close_grad(leaves[2].grad, want_q[1], dtype, "dwq")
+    _close_grad(leaves[3].grad, want_k[1], dtype, "dwk")
+    # q alone through the raw call: the same dq bits as in the joint launch (the weight gradient's rows
+    # are shared out over the workgroups differently, so its sum runs in another order)
+    dq, _, dwq, _ = hip_rope.rope_norm_bwd_raw(gq, None, q, None, pos, q_norm_weight=wq)
+    assert torch.equal(dq, leaves[0].grad) and rel_l2(dwq, want_q[1].float()) <= 2e-3
+    # a tensor without a weight gets the plain inverse rotation
+    dq2, dk2, dwq2, dwk2 = hip_rope.rope_norm_bwd_raw(gq, gk, q, k, pos, q_norm_weight=wq)
+    assert dwk2 is None and torch.equal(dq2, dq) and rel_l2(dwq2, dwq) <= 1e-5
+    assert torch.equal(dk2, hip_rope.rope_raw(None, gk, pos, inverse=True)[1])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_expert_norm_rotary_tables_gradients(dtype):
+    """cosmos3's expert: q_norm / k_norm and apply_rotary_pos_emb (qwen3vl_with_expert.py:217-224), trained;
+    head-major views of (b, s, h, d) projections, as the module makes them."""
+    b, h, hkv, s, d = 2, 16, 8, 50, 128
+    q_bshd, k_bshd = g(randn((b, s, h, d), dtype, 1) * 2.0), g(randn((b, s, hkv, d), dtype, 2) * 0.5)
+    wq, wk = g(1.0 + randn((d,), torch.float32, 3) * 0.2), g(1.0 + randn((d,), torch.float32, 4) * 0.2)
+    gq, gk = g(randn((b, h, s, d), dtype, 5)), g(randn((b, hkv, s, d), dtype, 6))
+    cos, sin = oracle.rope_tables(g(positions(b, s, 7)), d, 1_000_000, dtype)
+
+    def run(fn):
+        leaves = [t.clone().requires_grad_(True) for t in (q_bshd, k_bshd, wq, wk)]
+        qo, ko = fn(leaves[0].transpose(1, 2), leaves[1].transpose(1, 2), cos, sin, q_norm_weight=leaves[2],
+                    k_norm_weight=leaves[3], norm_eps=1e-6)
+        torch.autograd.backward([qo, ko], [gq, gk])
+        return [t.grad for t in leaves]
+
+    got = run(hip_rope.apply_rotary_pos_emb)
+    want_q = oracle.norm_rope_backward(q_bshd.transpose(1, 2), wq, gq, kind="qwen3", cos=cos, sin=sin)
+    want_k = oracle.norm_rope_backward(k_bshd.transpose(1, 2), wk, gk, kind="qwen3", cos=cos, sin=sin)
+    _close_grad(got[0], want_q[0].transpose(1, 2), dtype, "dq")
+    _close_grad(got[1], want_k[0].transpose(1, 2), dtype, "dk")
+    for a, e, name in ((got[2], want_q[1], "dwq"), (got[3], want_k[1], "dwk")):
+        r = rel_l2(a, e)
+        assert r <= (1e-5 if dtype == torch.float32 else 2e-3), f"{name}: rel-L2 {r:.3e}"
+    traced = run(torch.compile(hip_rope.apply_rotary_pos_emb, backend="aot_eager", fullgraph=True))
+    for a, e in zip(traced, got):
+        assert torch.equal(a, e)
+
+
+def test_norm_rope_gradient_argument_errors():
+    q = g(randn((1, 4, 2, 64), torch.bfloat16, 1)).requires_grad_(True)
+    k = g(randn((1, 4, 1, 64), torch.bfloat16, 2)).requires_grad_(True)
+    w = g(torch.zeros(64))
+    pos = g(torch.zeros(1, 4, dtype=torch.long))
+    with pytest.raises(RuntimeError, match="both norm weights"):
+        hip_rope.apply_rope_qk(q, k, pos, q_norm_weight=w)
+    with pytest.raises(RuntimeError, match="power of two|head_dim"):
+        x = g(randn((1, 4, 2, 96), torch.bfloat16, 1))
+        hip_rope.rope_norm_bwd_raw(x, None, x, None, pos, q_norm_weight=g(torch.zeros(96)))
+
+
 def test_rope_argument_errors():
     x = g(randn((1, 4, 2, 64), torch.bfloat16, 1))
     pos = g(torch.zeros(1, 4, dtype=torch.long))

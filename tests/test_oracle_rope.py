@@ -144,3 +144,56 @@ def test_expert_rms_norm_closed_form_and_roundings():
     normed = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16()
     assert torch.equal(rope.expert_rms_norm(xb, wb), (wb.float() * normed.float()).bfloat16())
     assert rope.expert_rms_norm(xb, w).dtype == torch.bfloat16  # fp32 weight on a bf16 input
+
+
+def _forward64(kind, x, w, angle):
+    """Norm then rotation in float64, written out: ``x (..., D)``, ``angle (..., D/2)``."""
+    half = x.shape[-1] // 2
+    r = 1.0 / torch.sqrt((x * x).mean(-1, keepdim=True) + 1e-6)
+    y = x * r * ((1.0 + w) if kind == "gemma3" else w)
+    lo, hi = y[..., :half], y[..., half:]
+    c, s = torch.cos(angle), torch.sin(angle)
+    return torch.cat([lo * c - hi * s, hi * c + lo * s], -1)
+
+
+def test_norm_rope_gradients_against_finite_differences():
+    """The gradient the fused backward is held to: autograd through the oracle's norm and rotation, checked
+    here against central differences of a float64 restatement of the forward (which the forward tests
+    above tie to the oracle).  A dropped mean term, a wrong sign of the inverse rotation or a missing
+    ``1 +`` on Gemma-3's weight each fail it."""
+    b, length, h, d = 2, 5, 3, 32
+    pos = torch.randint(0, 50, (b, length), generator=torch.Generator().manual_seed(1))
+    x = randn((b, length, h, d), torch.float32, 2) * 1.5
+    w = randn((d,), torch.float32, 3) * 0.3
+    go = randn((b, length, h, d), torch.float32, 4)
+    timescale = 10_000.0 ** ((2.0 / d) * torch.arange(d // 2, dtype=torch.float64))
+    angle = (pos.double().unsqueeze(-1) / timescale).unsqueeze(-2)  # (B, L, 1, D/2)
+    cos, sin = rope.rope_tables(pos, d, 10_000)
+    picks = torch.randint(0, x.numel(), (24,), generator=torch.Generator().manual_seed(5)).tolist()
+    for kind in ("gemma3", "qwen3"):
+        wk = w if kind == "gemma3" else 1.0 + w
+        if kind == "gemma3":
+            fwd = rope.apply_rope(rope.gemma3_rms_norm(x, wk), pos)
+            dx, dw = rope.norm_rope_backward(x, wk, go, kind=kind, positions=pos)
+        else:
+            xt, gt = x.transpose(1, 2).contiguous(), go.transpose(1, 2).contiguous()
+            fwd = rope.apply_rotary_pos_emb(rope.expert_rms_norm(xt, wk), xt[:, :0], cos, sin)[0].transpose(1, 2)
+            dx, dw = rope.norm_rope_backward(xt, wk, gt, kind=kind, cos=cos, sin=sin)
+            dx = dx.transpose(1, 2)
+        assert rel_l2(fwd, _forward64(kind, x.double(), wk.double(), angle)) <= 1e-6
+
+        def loss(xv, wv):
+            return float((_forward64(kind, xv, wv, angle) * go.double()).sum())
+
+        step = 1e-6
+        for at in picks:
+            e = torch.zeros(x.numel(), dtype=torch.float64)
+            e[at] = step
+            e = e.view_as(x)
+            fd = (loss(x.double() + e, wk.double()) - loss(x.double() - e, wk.double())) / (2 * step)
+            assert abs(fd - float(dx.flatten()[at])) <= 2e-4 * max(1.0, abs(fd)), (kind, at, fd)
+        for at in range(0, d, 5):
+            e = torch.zeros(d, dtype=torch.float64)
+            e[at] = step
+            fd = (loss(x.double(), wk.double() + e) - loss(x.double(), wk.double() - e)) / (2 * step)
+            assert abs(fd - float(dw[at])) <= 2e-4 * max(1.0, abs(fd)), (kind, "w", at, fd)
