@@ -243,7 +243,8 @@ size_t bcattn_bwd_workspace_bytes(const bcattn_bwd_params *p) {
   if (p == nullptr || p->B <= 0) return 0;
   return summary_bytes(p->B, p->Sk, p->Sk) + merged_bytes(p->B, p->Sk, p->Sk) +
          summary_bytes(p->B, p->Sq, p->Sq) + merged_bytes(p->B, p->Sq, p->Sq) +
-         2 * align256((size_t)p->B * p->H * pad64(p->Sq) * sizeof(float));
+         2 * align256((size_t)p->B * p->H * pad64(p->Sq) * sizeof(float)) +
+         (p->Hkv > 0 ? bwd_dkv_part_bytes(p->B, p->Sq, p->Sk, p->Hkv, p->H / p->Hkv, p->D, p->dtype) : 0);
 }
 
 int bcattn_fwd(const bcattn_fwd_params *p, void *stream) {
@@ -358,7 +359,7 @@ int bcattn_bwd(const bcattn_bwd_params *p, void *stream) {
   a.scale = p->scale;
   a.stages = p->stages & (BCATTN_BWD_DELTA | BCATTN_BWD_DQ | BCATTN_BWD_DKV);
   if (a.stages == 0) a.stages = BCATTN_BWD_DELTA | BCATTN_BWD_DQ | BCATTN_BWD_DKV;
-  // Backward workspace: [key summaries][key ids][query summaries][query ids][delta][log2e*LSE].
+  // Backward workspace: [key summaries][key ids][query summaries][query ids][delta][log2e*LSE][dK/dV partial sums].
   char *ws = reinterpret_cast<char *>(p->workspace);
   tile_summary_t *ks = reinterpret_cast<tile_summary_t *>(ws);
   ws += summary_bytes(a.B, a.Sk, a.Sk);
@@ -371,6 +372,9 @@ int bcattn_bwd(const bcattn_bwd_params *p, void *stream) {
   a.delta = reinterpret_cast<float *>(ws);
   ws += align256((size_t)a.B * a.H * a.Sq_pad * sizeof(float));
   a.lse2 = reinterpret_cast<float *>(ws);
+  ws += align256((size_t)a.B * a.H * a.Sq_pad * sizeof(float));
+  a.dkv_splits = bwd_dkv_splits(a.B, a.Sq, a.Sk, a.Hkv, a.G, p->D, p->dtype);
+  a.dkv_part = reinterpret_cast<float *>(ws);
   a.ksum = ks, a.qsum = qs, a.kbm = km, a.qbm = qm;
   if (!p->summary_ready &&
       ((rc = launch_summary(p->k_blk, p->k_valid, a.B, a.Sk, a.Sk, kIntMax, ks, km, st)) ||

@@ -307,12 +307,15 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, const unsigned bl
 
   const int Sk = a.Sk, Sq = a.Sq, Sqp = a.Sq_pad;
   const int nkt = (Sk + BK - 1) / BK;
-  const int nitems = nkt * a.Hkv * a.B;
+  const int HS = a.dkv_splits;  // workgroups that share this key block's query heads
+  const int nitems = nkt * a.Hkv * a.B * HS;
   int bid = xcd_item(block, nitems);
   if (bid >= nitems) return;
+  // (division results live in vector registers; say that they are uniform)
+  const int sp = __builtin_amdgcn_readfirstlane(bid % HS);
+  bid /= HS;
   const int kt = __builtin_amdgcn_readfirstlane(bid % nkt);
   bid /= nkt;
-  // (division results live in vector registers; say that they are uniform)
   const int hk = __builtin_amdgcn_readfirstlane(bid % a.Hkv);
   const int b = __builtin_amdgcn_readfirstlane(bid / a.Hkv);
 
@@ -351,8 +354,11 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, const unsigned bl
   __syncthreads();
 
   // Iterations run over (query head of the group, query tile), head-major; an iteration
-  // index is head << 16 | tile, so neither part needs a division.
-  const int nit = (kmin_g == kIntMax) ? 0 : a.G << 16;
+  // index is head << 16 | tile, so neither part needs a division.  This workgroup's heads:
+  // [sp, sp + 1) * G / HS.
+  const int gper = a.G / HS;
+  const int it0 = (sp * gper) << 16;
+  const int nit = (kmin_g == kIntMax) ? it0 : ((sp + 1) * gper) << 16;
 
   const e16_t *qb0 = reinterpret_cast<const e16_t *>(a.q.ptr) + b * a.q.sb + (int64_t)hk * a.G * a.q.sh;
   const e16_t *gb0 =
@@ -561,9 +567,27 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, const unsigned bl
   };
 
   settle_loads();
-  tile_pipeline<NS, LPT, LPT>(0, nit, find, issue, compute);
+  tile_pipeline<NS, LPT, LPT>(it0, nit, find, issue, compute);
 
-  if (jok) {
+  if (jok && HS > 1) {
+    // this workgroup's share of the sums, fp32, for bwd_dkv_reduce_kernel
+    const int64_t per = (int64_t)a.B * Sk * a.Hkv * D;
+    float *pk = a.dkv_part + sp * per + (((int64_t)b * Sk + j) * a.Hkv + hk) * D;
+    float *pv = pk + HS * per;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        f32x4 wk, wv;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          if (WANT_DK) wk[x] = dk[db][4 * r4 + x] * a.scale;
+          if (WANT_DV) wv[x] = dv[db][4 * r4 + x];
+        }
+        if (WANT_DK) *reinterpret_cast<f32x4 *>(pk + 32 * db + 8 * r4 + 4 * hh) = wk;
+        if (WANT_DV) *reinterpret_cast<f32x4 *>(pv + 32 * db + 8 * r4 + 4 * hh) = wv;
+      }
+  } else if (jok) {
     e16_t *dkp = reinterpret_cast<e16_t *>(a.dk) + b * a.dk_sb + (int64_t)j * a.dk_ss + hk * a.dk_sh;
     e16_t *dvp = reinterpret_cast<e16_t *>(a.dv) + b * a.dv_sb + (int64_t)j * a.dv_ss + hk * a.dv_sh;
 #pragma unroll
@@ -586,6 +610,41 @@ template <int D, int NW, int MODE>
 __global__ __launch_bounds__(64 * NW) void bwd_dkv_kernel(const BwdArgs a) {
   warm_kernel_arguments<sizeof(BwdArgs)>();
   bwd_dkv_body<D, NW, MODE>(a, blockIdx.x);
+}
+
+// Adds the dkv_splits partial sums of every dK / dV element in the order of the splits (fixed:
+// bit-repeatable), rounds once and stores: one thread per four elements.
+template <int D>
+__global__ __launch_bounds__(256) void bwd_dkv_reduce_kernel(const BwdArgs a) {
+  constexpr int LP = D / 4;
+  const int64_t rows = (int64_t)a.B * a.Sk * a.Hkv;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t row = idx / LP;
+  const int c = (int)(idx - row * LP);
+  if (row >= rows) return;
+  const int hk = (int)(row % a.Hkv);
+  const int64_t bj = row / a.Hkv;
+  const int j = (int)(bj % a.Sk), b = (int)(bj / a.Sk);
+  const int64_t per = rows * D;
+  const float *pk = a.dkv_part + row * D + 4 * c, *pv = pk + a.dkv_splits * per;
+  f32x4 sk = {0.f, 0.f, 0.f, 0.f}, sv = {0.f, 0.f, 0.f, 0.f};
+  for (int sp = 0; sp < a.dkv_splits; ++sp) {
+    const f32x4 xk = *reinterpret_cast<const f32x4 *>(pk + sp * per);
+    const f32x4 xv = *reinterpret_cast<const f32x4 *>(pv + sp * per);
+#pragma unroll
+    for (int x = 0; x < 4; ++x) sk[x] += xk[x], sv[x] += xv[x];
+  }
+  e16x4 wk, wv;
+#pragma unroll
+  for (int x = 0; x < 4; ++x) wk[x] = (e16_t)sk[x], wv[x] = (e16_t)sv[x];
+  *reinterpret_cast<e16x4 *>(reinterpret_cast<e16_t *>(a.dk) + b * a.dk_sb + (int64_t)j * a.dk_ss + hk * a.dk_sh + 4 * c) = wk;
+  *reinterpret_cast<e16x4 *>(reinterpret_cast<e16_t *>(a.dv) + b * a.dv_sb + (int64_t)j * a.dv_ss + hk * a.dv_sh + 4 * c) = wv;
+}
+
+template <int D>
+static void launch_dkv_reduce(const BwdArgs &a, hipStream_t st) {
+  const int64_t threads = (int64_t)a.B * a.Sk * a.Hkv * (D / 4);
+  hipLaunchKernelGGL(bwd_dkv_reduce_kernel<D>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, a);
 }
 
 // ---- dK / dV with paired waves --------------------------------------------------------
@@ -1120,7 +1179,7 @@ static int launch_dkv(const BwdArgs &a, hipStream_t st) {
   if (!needed_table_fits(dkv_smem_bytes<D>(), a.Sq_pad / 64)) return BCATTN_ERR_UNSUPPORTED;
   const size_t smem = dkv_smem_bytes<D>() + needed_table_bytes(a.Sq_pad / 64);
   const int nkt = (a.Sk + 32 * NW - 1) / (32 * NW);
-  hipLaunchKernelGGL((bwd_dkv_kernel<D, NW, MODE>), dim3(xcd_grid((unsigned)(nkt * a.Hkv * a.B))),
+  hipLaunchKernelGGL((bwd_dkv_kernel<D, NW, MODE>), dim3(xcd_grid((unsigned)(nkt * a.Hkv * a.B * a.dkv_splits))),
                      dim3(64 * NW), smem, st, a);
   return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
 }
@@ -1152,7 +1211,10 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
   const unsigned ndq = xcd_grid((unsigned)((R + 32 * NWQ - 1) / (32 * NWQ) * a.Hkv * a.B));
   const size_t smem_q = dq_smem_bytes<D>() + needed_table_bytes((a.Sk + 63) / 64);
   constexpr int kKeysPerGroup = 32 * (PAIRS > 0 ? PAIRS : NWK);
-  const unsigned ndkv = xcd_grid((unsigned)((a.Sk + kKeysPerGroup - 1) / kKeysPerGroup * a.Hkv * a.B));
+  const unsigned ndkv =
+      xcd_grid((unsigned)((a.Sk + kKeysPerGroup - 1) / kKeysPerGroup * a.Hkv * a.B * (PAIRS > 0 ? 1 : a.dkv_splits)));
+  if (PAIRS > 0 && a.dkv_splits != 1) return BCATTN_ERR_LAUNCH;  // (the paired kernel takes no split)
+  const bool reduce = (a.stages & BCATTN_BWD_DKV) && a.dkv_splits > 1;
   const bool both = (a.stages & BCATTN_BWD_DQ) && (a.stages & BCATTN_BWD_DKV);
   if (both && !serial_backward()) {
     if constexpr (PAIRS > 0) {
@@ -1169,6 +1231,7 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
       hipLaunchKernelGGL((bwd_dkv1_dq_kernel<D, NWQ, SPLIT>), dim3((SPLIT ? 2 : 1) * ndkv + ndq), dim3(64 * NWQ),
                          smem_kv > smem_q ? smem_kv : smem_q, st, a, ndkv);
     }
+    if (reduce) launch_dkv_reduce<D>(a, st);
     return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;
   }
   int rc = BCATTN_OK;
@@ -1180,6 +1243,7 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
     } else {
       rc = launch_dkv<D, NWK, kModeBoth>(a, st);
     }
+    if (!rc && reduce) launch_dkv_reduce<D>(a, st);
   }
   if (!rc && (a.stages & BCATTN_BWD_DQ))
     hipLaunchKernelGGL((bwd_dq_kernel<D, NWQ>), dim3(ndq), dim3(64 * NWQ), smem_q, st, a);

@@ -168,7 +168,37 @@ struct BwdArgs {
   int Sq_pad;  // Sq rounded up to whole 64-row tiles
   float scale;
   int stages;  // bit set of bcattn_bwd_stage, never 0 here
+  // dK/dV of few, long workgroups (small batch, one kv head): the query heads of a group are shared out
+  // over dkv_splits workgroups per key block, which leave fp32 partial sums in dkv_part
+  // ([dK | dV][split][B][Sk][Hkv][D]) that a second kernel adds in a fixed order.  1: no split.
+  int dkv_splits;
+  float *dkv_part;
 };
+
+// How many workgroups share a key block's query heads in the 16-bit dK/dV kernels (a divisor of G).  The
+// kernels take 128 keys per workgroup; a launch of fewer than kDkvFill of them leaves most of the chip idle
+// for the length of one workgroup's walk over G heads x all query tiles.  The paired-wave kernel (head_dim
+// 128, long rows) is not split: its launches are large.
+constexpr int kDkvFill = 128;
+inline int bwd_dkv_splits(int B, int Sq, int Sk, int Hkv, int G, int D, int dtype) {
+  if (dtype == BCATTN_F32 || G <= 1) return 1;
+  if (D == 128 && (int64_t)G * Sq >= 1024) return 1;
+  const int64_t base = (int64_t)((Sk + 127) / 128) * Hkv * B;
+  if (base >= kDkvFill) return 1;
+  const int nqt = (Sq + 63) / 64;
+  int best = 1;
+  for (int d = 2; d <= G; ++d) {
+    if (G % d) continue;
+    if ((G / d) * nqt < 4) break;  // a workgroup keeps at least four tiles of work
+    best = d;
+    if (base * d >= kDkvFill) break;
+  }
+  return best;
+}
+inline size_t bwd_dkv_part_bytes(int B, int Sq, int Sk, int Hkv, int G, int D, int dtype) {
+  const int sp = bwd_dkv_splits(B, Sq, Sk, Hkv, G, D, dtype);
+  return sp > 1 ? 2 * (size_t)sp * B * Sk * Hkv * D * sizeof(float) : 0;
+}
 
 struct RopeArgs {
   TensorArg q, k, q_out, k_out;  // a null ptr skips the tensor

@@ -161,7 +161,29 @@ def _check(rc: int, lib) -> None:
 
 
 def _stream(dev: torch.device) -> int:
-    return torch.cuda.current_stream(dev).cuda_stream
+    """The raw handle of torch's current stream on ``dev`` (no Stream object is built: this sits on
+    the path of every call)."""
+    return torch._C._cuda_getCurrentRawStream(dev.index if dev.index is not None else torch.cuda.current_device())
+
+
+class _on_device:
+    """``torch.cuda.device(dev)`` where ``dev`` is not the current device, nothing otherwise (the guard
+    costs more than the rest of a call's Python on the usual one-GPU process)."""
+
+    __slots__ = ("guard",)
+
+    def __init__(self, dev: torch.device):
+        idx = dev.index
+        self.guard = torch.cuda.device(dev) if idx is not None and idx != torch.cuda.current_device() else None
+
+    def __enter__(self):
+        if self.guard is not None:
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            self.guard.__exit__(*exc)
+        return False
 
 
 def _check_inputs(q, k, v):
@@ -284,7 +306,7 @@ def forward_raw(
     p.summary_ready = 1 if summary_ready else 0
     p.kv_share = share
     if static_scratch:
-        with torch.cuda.device(q.device):
+        with _on_device(q.device):
             _check(lib.bcattn_fwd_kvcache_static(ctypes.byref(p), _stream(q.device)), lib)
         return out, lse
     size_fn = lib.bcattn_fwd_kvcache_workspace_bytes if kvcache else lib.bcattn_fwd_workspace_bytes
@@ -302,7 +324,7 @@ def forward_raw(
             raise RuntimeError("summary_ready needs the workspace of the earlier call")
         workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
     p.workspace, p.workspace_bytes = workspace.data_ptr(), workspace.numel()
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         fn = lib.bcattn_fwd_kvcache if kvcache else lib.bcattn_fwd
         _check(fn(ctypes.byref(p), _stream(q.device)), lib)
     if slot is not None:
@@ -381,7 +403,7 @@ def backward_raw(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale
             raise RuntimeError("this call needs the workspace an earlier call filled")
         workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
     p.workspace, p.workspace_bytes = workspace.data_ptr(), workspace.numel()
-    with torch.cuda.device(q.device):
+    with _on_device(q.device):
         _check(lib.bcattn_bwd(ctypes.byref(p), _stream(q.device)), lib)
     if slot is not None:
         slot["fwd"] = slot["bwd"] = True  # the backward's summary pass covers the keys as well
@@ -576,8 +598,12 @@ def flash_attn_blockmask(
         if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
             return _HeldBlockMask.apply(q, k, v, float(scale), block_ids)
         return forward_raw(q, k, v, *block_ids, scale, want_lse=False, block_ids=block_ids)[0]
-    if _needs_graph(q, k, v):
+    if torch.compiler.is_compiling():
         return _op_fwd(q, k, v, q_blk, k_blk, q_valid, k_valid, float(scale))[0]
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v)):
+        # eager autograd: the plain Function costs a third of the dispatch of the traceable op, and a
+        # holder made for this call lets its backward use the forward's key summary
+        return _HeldBlockMask.apply(q, k, v, float(scale), BlockIds(q_blk, k_blk, q_valid, k_valid))
     return forward_raw(q, k, v, q_blk, k_blk, q_valid, k_valid, scale, want_lse=False)[0]
 
 

@@ -20,7 +20,7 @@ import ctypes
 import torch
 
 from .flash_attn_hip import _loader
-from .flash_attn_hip import _check, _DTYPES, _stream, _t4
+from .flash_attn_hip import _check, _DTYPES, _on_device, _stream, _t4
 
 _timescales: dict[tuple, torch.Tensor] = {}
 _NORM_KINDS = {"gemma3": 0, "qwen3": 1}  # enum bcattn_norm_kind
@@ -143,7 +143,7 @@ def rope_raw(
     p.H = q.shape[2] if q is not None else 0
     p.Hkv = k.shape[2] if k is not None else 0
     p.n_axes, p.dtype, p.inverse, p.norm_eps = n_axes, code, 1 if inverse else 0, float(norm_eps)
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         _check(lib.bcattn_rope(ctypes.byref(p), _stream(x.device)), lib)
     return (q_out if q is not None else None), (k_out if k is not None else None)
 
@@ -208,7 +208,7 @@ def rope_norm_bwd_raw(
     blocks = int(lib.bcattn_rope_norm_bwd_blocks(ctypes.byref(p)))
     partial = torch.empty((max(blocks, 1), 2, d), dtype=torch.float32, device=x.device)
     p.dw_partial = partial.data_ptr()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         _check(lib.bcattn_rope_norm_bwd(ctypes.byref(p), _stream(x.device)), lib)
     dw = partial[:blocks].sum(0)  # (2, D): one fixed-order reduction for both weights
     if stacked:

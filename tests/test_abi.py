@@ -72,6 +72,13 @@ def test_workspace_queries_run_without_a_gpu():
     bp = _loader.BwdParams()
     bp.B, bp.Sq, bp.Sk, bp.H, bp.Hkv, bp.D = 2, 100, 130, 4, 2, 128
     assert lib.bcattn_bwd_workspace_bytes(ctypes.byref(bp)) >= 2 * 4 * 100 * 4
+    # One sample, one kv head: the 8 key blocks' dK/dV work is shared out over the 8 query heads, and the
+    # workspace grows by the fp32 partial sums, 2 (dK, dV) x 8 x Sk x D floats; with 8 kv heads (no groups
+    # to share out) it does not.
+    bp.B, bp.Sq, bp.Sk, bp.H, bp.Hkv, bp.D, bp.dtype = 1, 1024, 1024, 8, 1, 256, _loader.DTYPE_BF16
+    shared = lib.bcattn_bwd_workspace_bytes(ctypes.byref(bp))
+    bp.Hkv = 8
+    assert shared - lib.bcattn_bwd_workspace_bytes(ctypes.byref(bp)) == 2 * 8 * 1024 * 256 * 4
 
 
 def test_argument_errors_are_reported_not_crashed():

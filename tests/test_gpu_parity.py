@@ -300,6 +300,39 @@ def test_other_head_dims_the_reference_accepts(dtype, head_dim):
         assert rel_l2(got, want) <= 1e-2, name
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("b,sq,cross,h,hkv,d,pattern", [
+    (1, 520, 0, 8, 1, 256, "prefixlm"),      # the reference harness's geometry: 5 key blocks, 8 heads each
+    (2, 333, 0, 8, 2, 64, "multiblock"),     # groups of 4 heads
+    (1, 200, 70, 16, 4, 128, "causal"),      # the single-wave head_dim 128 kernel (short rows), cached keys in front
+    (1, 300, 0, 6, 1, 256, "prefixlm"),      # a group size that is no power of two
+    (3, 150, 0, 4, 1, 256, "bidir"),
+])
+def test_small_batch_backward_shares_heads_over_workgroups(dtype, b, sq, cross, h, hkv, d, pattern):
+    """Few (batch, kv head, key block) workgroups: the dK/dV kernels share a group's query heads out over
+    several workgroups and a second kernel adds their fp32 partial sums.  Same bar as the other
+    backward tests; bit-repeatable; the gradients of one stage asked alone are the same bits."""
+    ids = make_blocks(b, sq, pattern, cross=cross, pad_tail=9)
+    q, k, v = _qkv(b, sq, cross + sq, h, hkv, d, dtype, seed=5)
+    go = randn((b, sq, h, d), dtype, 9)
+    scale = d**-0.5
+    out, dq, dk, dv = _fwd_bwd(q, k, v, go, ids, scale)
+    _, rq, rk, rv = eager.eager_grads(q.float(), k.float(), v.float(), go.float(), *ids, scale)
+    qm = ids[2][:, :, None, None]
+    for got, ref, name in ((dq.float() * qm, rq * qm, "dq"), (dk.float(), rk, "dk"), (dv.float(), rv, "dv")):
+        torch.testing.assert_close(got, ref, atol=5e-2, rtol=5e-2)
+        assert rel_l2(got, ref) <= (1e-2 if dtype == torch.bfloat16 else 2e-3), name
+    again = _fwd_bwd(q, k, v, go, ids, scale)
+    for x, y in zip((out, dq, dk, dv), again):
+        assert torch.equal(x, y)
+    # dK / dV alone (the row sums first, then only that stage)
+    gi = [g(t) for t in ids]
+    o2, lse = fa.forward_raw(g(q), g(k), g(v), *gi, scale)
+    _, dk2, dv2 = fa.backward_raw(g(go), g(q), g(k), g(v), o2, lse, *gi, scale,
+                                  stages=fa._loader.BWD_DELTA | fa._loader.BWD_DKV)
+    assert torch.equal(dk2.cpu(), dk) and torch.equal(dv2.cpu(), dv)
+
+
 def test_backward_is_bit_repeatable():
     b, sq, h, hkv, d = 2, 300, 8, 2, 128
     ids = make_blocks(b, sq, "multiblock", pad_tail=17)
