@@ -518,35 +518,55 @@ def _kvc_setup(ctx, inputs, output):
     ctx.scale = scale
 
 
+def _kvc_grads(bwd, d_out, q, k_cache, v_cache, k_new, v_new, out, lse, q_blk, k_blk, q_valid, k_valid, scale, need):
+    """Gradients of the KV-cached call, ``need`` = which of (q, k_cache, v_cache, k_new, v_new) want one.
+    ``bwd(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale, stages) -> (dq, dk, dv)``.
+
+    With LSE and the row sums of O * dO taken over all keys, every term of the backward is a sum over keys:
+    the two segments go through the backward one after the other, each with its own slice of the key ids,
+    and only dQ has to be added up.  So the segments are never joined (the copy of the whole cache per layer
+    that the forward avoids), and a segment nobody wants gradients for costs its dQ share only (training
+    with a cache is the knowledge-insulation case, ``src/opentau/policies/pi05/modeling_pi05.py:1752-1757``,
+    whose cached K/V are detached).  A cache shared by several batch entries takes the joined path: its
+    gradient is a sum over those entries."""
+    n0, n1 = k_cache.shape[1], k_new.shape[1]
+    share = q.shape[0] // k_cache.shape[0]
+    want_q, want_c, want_n = need[0], need[1] or need[2], need[3] or need[4]
+    if share > 1 or n0 == 0 or n1 == 0:
+        if share > 1:  # a shared cache entry collects the gradients of all the entries that read it
+            k_cache, v_cache = (t.repeat_interleave(share, dim=0) for t in (k_cache, v_cache))
+        k = torch.cat([k_cache, k_new], dim=1)
+        v = torch.cat([v_cache, v_new], dim=1)
+        dq, dk, dv = bwd(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale,
+                         _wanted_stages(want_q, want_c or want_n))
+        dkc = dvc = None
+        if want_c:
+            dkc, dvc = dk[:, :n0], dv[:, :n0]
+            if share > 1:
+                dkc, dvc = (t.reshape(-1, share, *t.shape[1:]).float().sum(1).to(t.dtype) for t in (dkc, dvc))
+        return dq, dkc, dvc, dk[:, n0:], dv[:, n0:]
+    dq = dkc = dvc = dkn = dvn = None
+    if want_q or want_c:
+        dq, dkc, dvc = bwd(d_out, q, k_cache, v_cache, out, lse, q_blk, k_blk[:, :n0], q_valid, k_valid[:, :n0], scale,
+                           _wanted_stages(want_q, want_c))
+    if want_q or want_n:
+        dq1, dkn, dvn = bwd(d_out, q, k_new, v_new, out, lse, q_blk, k_blk[:, n0:], q_valid, k_valid[:, n0:], scale,
+                            _wanted_stages(want_q, want_n))
+        if want_q:
+            dq = (dq.float() + dq1.float()).to(dq.dtype)
+    return dq, dkc, dvc, dkn, dvn
+
+
 def _kvc_backward(ctx, d_out, _d_lse):
-    # The backward kernels take the keys as one segment, so the two are joined here: a copy of
-    # B*Sk*Hkv*D elements per layer, against attention work that grows with Sq*Sk*H*D.  (Training
-    # with a cache is the knowledge-insulation case, whose cached K/V are detached: then only dQ
-    # and the new keys' gradients are wanted, and with nothing wanted for K/V the dK/dV kernel is skipped.)
     q, k_cache, v_cache, k_new, v_new, out, lse, q_blk, k_blk, q_valid, k_valid = ctx.saved_tensors
     need = ctx.needs_input_grad
-    n0 = k_cache.shape[1]
-    share = q.shape[0] // k_cache.shape[0]
-    if share > 1:  # a shared cache entry collects the gradients of all the entries that read it
-        k_cache, v_cache = (t.repeat_interleave(share, dim=0) for t in (k_cache, v_cache))
-    k = torch.cat([k_cache, k_new], dim=1)
-    v = torch.cat([v_cache, v_new], dim=1)
-    stages = _wanted_stages(need[0], any(need[1:5]))
-    dq, dk, dv = _op_bwd(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, ctx.scale, stages)
-    dkc = dvc = None
-    if need[1] or need[2]:
-        dkc, dvc = dk[:, :n0], dv[:, :n0]
-        if share > 1:
-            dkc, dvc = (t.reshape(-1, share, *t.shape[1:]).float().sum(1).to(t.dtype) for t in (dkc, dvc))
+    dq, dkc, dvc, dkn, dvn = _kvc_grads(_op_bwd, d_out, q, k_cache, v_cache, k_new, v_new, out, lse, q_blk, k_blk,
+                                        q_valid, k_valid, ctx.scale, need)
     return (dq if need[0] else None, dkc if need[1] else None, dvc if need[2] else None,
-            dk[:, n0:] if need[3] else None, dv[:, n0:] if need[4] else None, None, None, None, None, None)
+            dkn if need[3] else None, dvn if need[4] else None, None, None, None, None, None)
 
 
 _op_fwd_kvcache.register_autograd(_kvc_backward, setup_context=_kvc_setup)
-
-
-def _needs_graph(*ts: torch.Tensor) -> bool:
-    return torch.compiler.is_compiling() or (torch.is_grad_enabled() and any(t.requires_grad for t in ts))
 
 
 class _HeldBlockMask(torch.autograd.Function):
@@ -572,6 +592,30 @@ class _HeldBlockMask(torch.autograd.Function):
         dq, dk, dv = backward_raw(d_out, q, k, v, out, lse, *ctx.held, ctx.scale, stages=stages, block_ids=ctx.held)
         return (dq if want_q else None, dk if ctx.needs_input_grad[1] else None,
                 dv if ctx.needs_input_grad[2] else None, None, None)
+
+
+class _HeldBlockMaskKvcache(torch.autograd.Function):
+    """The eager autograd path of the KV-cached call (the traced one is ``bcattn::fwd_kvcache``)."""
+
+    @staticmethod
+    def forward(ctx, q, k_cache, v_cache, k_new, v_new, scale, held):
+        out, lse = forward_raw(q, k_cache, v_cache, *held, scale, k_new, v_new, kvcache=True, block_ids=held)
+        ctx.save_for_backward(q, k_cache, v_cache, k_new, v_new, out, lse)
+        ctx.scale, ctx.held = scale, held
+        return out
+
+    @staticmethod
+    def backward(ctx, d_out):
+        q, k_cache, v_cache, k_new, v_new, out, lse = ctx.saved_tensors
+        need = ctx.needs_input_grad
+
+        def bwd(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale, stages):
+            return backward_raw(d_out, q, k, v, out, lse, q_blk, k_blk, q_valid, k_valid, scale, stages=stages)
+
+        dq, dkc, dvc, dkn, dvn = _kvc_grads(bwd, d_out, q, k_cache, v_cache, k_new, v_new, out, lse, *ctx.held,
+                                            ctx.scale, need)
+        return (dq if need[0] else None, dkc if need[1] else None, dvc if need[2] else None,
+                dkn if need[3] else None, dvn if need[4] else None, None, None)
 
 
 def flash_attn_blockmask(
@@ -634,11 +678,14 @@ def flash_attn_blockmask_kvcache(
     the ``n`` copies of the prefix cache that ``expand_kv_cache`` makes
     (``src/opentau/policies/candidates.py:114-127``).
     """
-    if block_ids is not None and not _needs_graph(q, k_cache, v_cache, k_new, v_new):
+    if torch.compiler.is_compiling():
+        return _op_fwd_kvcache(q, k_cache, v_cache, k_new, v_new, q_blk, k_blk, q_valid, k_valid, float(scale))[0]
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k_cache, v_cache, k_new, v_new)):
+        held = block_ids if block_ids is not None else BlockIds(q_blk, k_blk, q_valid, k_valid)
+        return _HeldBlockMaskKvcache.apply(q, k_cache, v_cache, k_new, v_new, float(scale), held)
+    if block_ids is not None:
         return forward_raw(q, k_cache, v_cache, *block_ids, scale, k_new, v_new, kvcache=True, want_lse=False,
                            block_ids=block_ids)[0]
-    if _needs_graph(q, k_cache, v_cache, k_new, v_new):
-        return _op_fwd_kvcache(q, k_cache, v_cache, k_new, v_new, q_blk, k_blk, q_valid, k_valid, float(scale))[0]
     return forward_raw(
         q, k_cache, v_cache, q_blk, k_blk, q_valid, k_valid, scale, k_new, v_new, kvcache=True, want_lse=False
     )[0]

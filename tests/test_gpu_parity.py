@@ -557,6 +557,42 @@ def test_kvcache_shared_gradients_sum_over_candidates():
         assert_close_bf16(a.float().cpu(), e.float().cpu(), name)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("insulated", [False, True])
+def test_kvcache_gradients_match_the_oracle_on_the_joined_keys(dtype, insulated):
+    """The training use of the cached call (pi0.5's suffix pass, ``pi05/modeling_pi05.py:1735-1767``): its
+    backward takes the two key segments one after the other and adds the dQ shares.  Against autograd
+    through the eager oracle on ``cat(cache, new)``; with the cache detached (knowledge insulation,
+    ``:1752-1757``) only q and the new keys get gradients."""
+    b, sq, h, hkv, d, cross = 2, 50, 8, 1, 256, 200
+    ids = make_blocks(b, sq, "prefixlm", cross=cross)
+    q, k, v = _qkv(b, sq, cross + sq, h, hkv, d, dtype, seed=11)
+    go = randn((b, sq, h, d), dtype, 12)
+    scale = d**-0.5
+    leaf = lambda t, grad=True: g(t).clone().requires_grad_(grad)  # noqa: E731
+    qq, kn, vn = leaf(q), leaf(k[:, cross:]), leaf(v[:, cross:])
+    kc, vc = leaf(k[:, :cross], not insulated), leaf(v[:, :cross], not insulated)
+    out = fa.flash_attn_blockmask_kvcache(qq, kc, vc, kn, vn, *[g(t) for t in ids], scale)
+    out.backward(g(go))
+    _, rq, rk, rv = eager.eager_grads(q.float(), k.float(), v.float(), go.float(), *ids, scale)
+    close = assert_close_f32 if dtype == torch.float32 else assert_close_bf16
+    close(qq.grad.float().cpu(), rq, "dq")
+    close(kn.grad.float().cpu(), rk[:, cross:], "dk_new")
+    close(vn.grad.float().cpu(), rv[:, cross:], "dv_new")
+    if insulated:
+        assert kc.grad is None and vc.grad is None
+    else:
+        close(kc.grad.float().cpu(), rk[:, :cross], "dk_cache")
+        close(vc.grad.float().cpu(), rv[:, :cross], "dv_cache")
+    # the traced form gives the same gradients
+    q2, kn2, vn2 = leaf(q), leaf(k[:, cross:]), leaf(v[:, cross:])
+    kc2, vc2 = leaf(k[:, :cross], not insulated), leaf(v[:, :cross], not insulated)
+    traced = torch.compile(fa.flash_attn_blockmask_kvcache, backend="aot_eager", fullgraph=True)
+    traced(q2, kc2, vc2, kn2, vn2, *[g(t) for t in ids], scale).backward(g(go))
+    for a, e in ((q2.grad, qq.grad), (kn2.grad, kn.grad), (vn2.grad, vn.grad), (kc2.grad, kc.grad)):
+        assert (a is None and e is None) or torch.equal(a, e)
+
+
 def test_kvcache_share_must_divide_batch():
     d = 64
     gi = [g(t) for t in make_blocks(3, 8, "prefixlm", cross=16)]
