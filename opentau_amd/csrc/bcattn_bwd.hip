@@ -462,25 +462,36 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, const unsigned bl
         if (WANT_DK) dp[mb] = mfma32(rowa.template read<Gt>(32 * mb, ks), vf[ks], dp[mb]);
       });
     };
-    auto softmax = [&](int mb) __attribute__((always_inline)) {
+    // The statistics of a half's queries (log2e * LSE, -delta, ids) are read into registers by a call
+    // of their own, placed in front of the products they are to run beside: the scheduler fills its
+    // groups in program order, and reads that come after a phase's operand reads in the source would be
+    // issued after them, with the softmax behind both.
+    struct Stats {
+      f32x4 lse[4], del[4];
+      i32x4 qb[4];
+    };
+    auto load_stats = [&](int mb, Stats &st) __attribute__((always_inline)) {
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const int q0 = 32 * mb + 8 * r4 + 4 * hh;
+        st.lse[r4] = *reinterpret_cast<const f32x4 *>(lse_s + q0);
+        if (WANT_DK) st.del[r4] = *reinterpret_cast<const f32x4 *>(delta_s + q0);
+        if (MASKED) st.qb[r4] = *reinterpret_cast<const i32x4 *>(qb_s + q0);
+      }
+    };
+    auto softmax = [&](int mb, const Stats &st) __attribute__((always_inline)) {
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         float p[8], ds[8];
 #pragma unroll
         for (int r2 = 0; r2 < 2; ++r2) {
           const int r4 = 2 * half + r2;
-          const int q0 = 32 * mb + 8 * r4 + 4 * hh;
-          const f32x4 lse4 = *reinterpret_cast<const f32x4 *>(lse_s + q0);
-          f32x4 del4 = {0.f, 0.f, 0.f, 0.f};
-          if (WANT_DK) del4 = *reinterpret_cast<const f32x4 *>(delta_s + q0);
-          i32x4 qb4 = {0, 0, 0, 0};
-          if (MASKED) qb4 = *reinterpret_cast<const i32x4 *>(qb_s + q0);
 #pragma unroll
           for (int x = 0; x < 4; ++x) {
-            float pv = fast_exp2(s[mb][4 * r4 + x] * c - lse4[x]);
-            if (MASKED && kb > qb4[x]) pv = 0.f;
+            float pv = fast_exp2(s[mb][4 * r4 + x] * c - st.lse[r4][x]);
+            if (MASKED && kb > st.qb[r4][x]) pv = 0.f;
             p[4 * r2 + x] = pv;
-            if (WANT_DK) ds[4 * r2 + x] = pv * (dp[mb][4 * r4 + x] + del4[x]);  // del4 holds -delta
+            if (WANT_DK) ds[4 * r2 + x] = pv * (dp[mb][4 * r4 + x] + st.del[r4][x]);  // del holds -delta
           }
         }
         if (WANT_DV) pb[mb][half] = pack8(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7]);
@@ -514,8 +525,10 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, const unsigned bl
     }
     __builtin_amdgcn_sched_barrier(0);
 
+    Stats st;
+    load_stats(0, st);
     phase_a(StageC<1>{});
-    softmax(0);
+    softmax(0, st);
     {
       constexpr int kAhead = NA < 4 ? NA : 4;
       __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
@@ -524,20 +537,24 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, const unsigned bl
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // next operand + statistics reads
         __builtin_amdgcn_sched_group_barrier(0x002, VA, 0);
+        __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);  // (the exponentials are a class of their own)
       }
     }
     __builtin_amdgcn_sched_barrier(0);
 
+    load_stats(1, st);
     phase_c(0);
-    softmax(1);
+    softmax(1, st);
     {
+      constexpr int NSTAT = 4 * (1 + (WANT_DK ? 1 : 0) + (MASKED ? 1 : 0));  // statistics reads of a half
       constexpr int kAhead = NC < 4 ? NC : 4;
-      __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, NSTAT + 2 * kAhead, 0);
 #pragma unroll
       for (int x = 0; x < NC; ++x) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 3, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
         __builtin_amdgcn_sched_group_barrier(0x002, VA, 0);
+        __builtin_amdgcn_sched_group_barrier(0x400, 1, 0);
       }
     }
     __builtin_amdgcn_sched_barrier(0);
