@@ -261,8 +261,9 @@ def bench_train(torch, fa, w, dev, steps, warmup):
 def bench_dispatch(torch, fa, w, dev, steps=20, warmup=3):
     """What the PyTorch-facing call adds to the raw C-ABI step: the same forward + backward through
     ``flash_attention_forward`` and autograd (outputs and gradients allocated by the framework), once
-    with a plain tuple of block ids (the traced custom ops; workspace and summaries per call) and once
-    with a ``BlockIds`` (workspace and summaries kept across calls), HIP-event median per step."""
+    with a plain tuple of block ids (workspace and summaries per call, the backward sharing the
+    forward's) and once with a ``BlockIds`` (workspace and summaries kept across calls), HIP-event
+    median per step."""
     from opentau_amd import attention
 
     plain = tuple(t.to(dev) for t in w.block_ids())
