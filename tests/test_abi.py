@@ -99,6 +99,15 @@ def test_argument_errors_are_reported_not_crashed():
     assert lib.bcattn_fwd(ctypes.byref(p), None) == _loader.ERR_INVALID  # null q
     assert b"null" in lib.bcattn_last_error()
     assert lib.bcattn_bwd(None, None) == _loader.ERR_INVALID
+    # the gradient of the norm + rotary call: argument checks come before anything touches a device
+    assert lib.bcattn_rope_norm_bwd(None, None) == _loader.ERR_INVALID
+    r = _loader.RopeNormBwdParams()
+    r.B, r.L, r.H, r.Hkv, r.D, r.n_axes, r.dtype = 1, 4, 2, 1, 96, 1, _loader.DTYPE_BF16
+    assert lib.bcattn_rope_norm_bwd(ctypes.byref(r), None) == _loader.ERR_UNSUPPORTED
+    assert b"power-of-two" in lib.bcattn_last_error()
+    r.D = 128
+    assert lib.bcattn_rope_norm_bwd(ctypes.byref(r), None) == _loader.ERR_INVALID  # no positions / tables
+    assert lib.bcattn_rope_norm_bwd_blocks(ctypes.byref(r)) == 0  # (no gradient tensors: nothing to launch)
 
 
 @pytest.mark.skipif(torch.cuda.is_available(), reason="checks the no-GPU behaviour")
