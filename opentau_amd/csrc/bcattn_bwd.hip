@@ -65,6 +65,13 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const BwdArgs a) {
 }
 
 // LDS stages: three where they fit in the 160 KB of a CU, else two.
+// Ends a step of a hand-ordered sequence: neither the compiler's code motion (the empty asm statement with
+// its memory clobber holds the LDS reads in place) nor the instruction scheduler moves anything across.
+__device__ __forceinline__ void pin_step() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+
 template <int D>
 struct BwdStages {
   static constexpr int value = D <= 128 ? 3 : 2;
@@ -206,25 +213,40 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a, const unsigned blo
       f32x16 s, dp = nd16;
 #pragma unroll
       for (int x = 0; x < 16; ++x) s[x] = 0.f;
-      constexpr int KB = 2;  // operand reads issued ahead of the products
-      static_for<DK / KB>([&](auto b_c) {
-        constexpr int k0 = decltype(b_c)::value * KB;
-        e16x8 fa[KB], fb[KB];
+      // Operand reads run KA (KC) products ahead in rings of registers, pinned step by step: left to
+      // the scheduler they end up one product ahead and every product waits out an LDS round trip.
+      constexpr int KA = 3, KC = 4;
+      e16x8 fa[KA], fb[KA];
 #pragma unroll
-        for (int ks = 0; ks < KB; ++ks) {
-          fa[ks] = rowa.template read<Kt>(32 * mb, k0 + ks);
-          fb[ks] = rowa.template read<Vt>(32 * mb, k0 + ks);
-        }
+      for (int i = 0; i < KA; ++i) {
+        fa[i] = rowa.template read<Kt>(32 * mb, i);
+        fb[i] = rowa.template read<Vt>(32 * mb, i);
+      }
+      pin_step();
+      static_for<DK>([&](auto ks_c) {
+        constexpr int ks = decltype(ks_c)::value;
         // the loads of the tile due in this step go out between the products of the first half
-        static_for<KB>([&](auto ks_c) {
-          if constexpr (mb == 0) parts_at_slot<k0 + decltype(ks_c)::value, DK, LPT>(bg);
-        });
-#pragma unroll
-        for (int ks = 0; ks < KB; ++ks) {
-          s = mfma32(fa[ks], qf[k0 + ks], s);
-          dp = mfma32(fb[ks], gof[k0 + ks], dp);
+        if constexpr (mb == 0) parts_at_slot<ks, DK, LPT>(bg);
+        s = mfma32(fa[ks % KA], qf[ks], s);
+        dp = mfma32(fb[ks % KA], gof[ks], dp);
+        // (the products are pure values to the compiler, which would sink them behind the last read:
+        // an empty asm statement that takes and returns the accumulators holds them in their step)
+        // (head_dim 256 keeps accumulators in the AGPR half of its register file)
+        if constexpr (D == 256)
+          asm volatile("" : "+a"(s), "+a"(dp));
+        else
+          asm volatile("" : "+v"(s), "+v"(dp));
+        if constexpr (ks + KA < DK) {
+          fa[ks % KA] = rowa.template read<Kt>(32 * mb, ks + KA);
+          fb[ks % KA] = rowa.template read<Vt>(32 * mb, ks + KA);
         }
+        pin_step();
       });
+      // the first transposed operands of the dQ products are on their way during the softmax
+      constexpr int NCS = 2 * DB;
+      e16x8 ta[KC];
+#pragma unroll
+      for (int i = 0; i < KC; ++i) ta[i] = tra.template read<Kt>(2 * mb + i / DB, i % DB);
       float ds[16];
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
@@ -240,14 +262,13 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a, const unsigned blo
       e16x8 dsb[2];
       dsb[0] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
       dsb[1] = pack8(ds[8], ds[9], ds[10], ds[11], ds[12], ds[13], ds[14], ds[15]);
-#pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        e16x8 ka[DB];
-#pragma unroll
-        for (int db = 0; db < DB; ++db) ka[db] = tra.template read<Kt>(2 * mb + half, db);
-#pragma unroll
-        for (int db = 0; db < DB; ++db) dq[db] = mfma32(ka[db], dsb[half], dq[db]);
-      }
+      pin_step();
+      static_for<NCS>([&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        dq[i % DB] = mfma32(ta[i % KC], dsb[i / DB], dq[i % DB]);
+        if constexpr (i + KC < NCS) ta[i % KC] = tra.template read<Kt>(2 * mb + (i + KC) / DB, (i + KC) % DB);
+        pin_step();
+      });
     });
   };
   auto compute = [&](auto stage_c, int t, auto bg) __attribute__((always_inline)) {
@@ -293,6 +314,10 @@ template <int D, int NW, int MODE>
 __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, const unsigned block) {
   using T = Tile<D>;
   constexpr bool WANT_DV = MODE != kModeDK, WANT_DK = MODE != kModeDV;
+#ifndef BCATTN_SEQ_HALVES
+#define BCATTN_SEQ_HALVES 1
+#endif
+  constexpr bool kSeqHalves = BCATTN_SEQ_HALVES && D == 256;
   constexpr int NT = 64 * NW, BK = 32 * NW;
   constexpr int DK = D / 16, DB = D / 32;
   constexpr int NS = BwdStages<D>::value;
@@ -512,6 +537,64 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, const unsigned bl
     constexpr int NC = 2 * DB * PER;                                  // products of one C phase
     constexpr int VA = (MASKED ? 9 : 7) * 16 / (NA < NC ? NA : NC) + 1;  // vector ALU instr. per product
 
+    if constexpr (kSeqHalves) {
+      // One half after the other: the products of S (and dP), the softmax on its own, the accumulating
+      // products.  Nothing of one half is held while the other is worked on, which leaves registers for
+      // operand reads KA / KC products ahead; those are written out as rings of registers and pinned
+      // step by step (left to the scheduler, the reads of the dK form end up one product ahead, each
+      // product waiting out a whole LDS round trip).
+      Stats st;
+      static_for<2>([&](auto mb_c) {
+        constexpr int mb = decltype(mb_c)::value;
+        constexpr int KA = 3, KC = 4;
+        load_stats(mb, st);
+        e16x8 fq[KA], fg[WANT_DK ? KA : 1];
+#pragma unroll
+        for (int i = 0; i < KA; ++i) {
+          fq[i] = rowa.template read<Qt>(32 * mb, i);
+          if (WANT_DK) fg[i] = rowa.template read<Gt>(32 * mb, i);
+        }
+#pragma unroll
+        for (int x = 0; x < 16; ++x) {
+          s[mb][x] = 0.f;
+          if constexpr (WANT_DK) dp[mb][x] = 0.f;
+        }
+        pin_step();
+        static_for<DK>([&](auto ks_c) {
+          constexpr int ks = decltype(ks_c)::value;
+          parts_at_slot<mb * DK + ks, 2 * DK, LPT>(bg);
+          s[mb] = mfma32(fq[ks % KA], kf[ks], s[mb]);
+          if (WANT_DK) dp[mb] = mfma32(fg[ks % KA], vf[ks], dp[mb]);
+          if constexpr (ks + KA < DK) {
+            fq[ks % KA] = rowa.template read<Qt>(32 * mb, ks + KA);
+            if (WANT_DK) fg[ks % KA] = rowa.template read<Gt>(32 * mb, ks + KA);
+          }
+          pin_step();
+        });
+        softmax(mb, st);
+        pin_step();
+        // accumulating products: step i is (16-query quarter i / DB of the half, head_dim block i % DB)
+        constexpr int NCS = 2 * DB;
+        e16x8 ta[WANT_DV ? KC : 1], tb[WANT_DK ? KC : 1];
+#pragma unroll
+        for (int i = 0; i < KC; ++i) {
+          if (WANT_DV) ta[i] = tra.template read<Gt>(2 * mb + i / DB, i % DB);
+          if (WANT_DK) tb[i] = tra.template read<Qt>(2 * mb + i / DB, i % DB);
+        }
+        pin_step();
+        static_for<NCS>([&](auto i_c) {
+          constexpr int i = decltype(i_c)::value;
+          if (WANT_DV) dv[i % DB] = mfma32(ta[i % KC], pb[mb][i / DB], dv[i % DB]);
+          if (WANT_DK) dk[i % DB] = mfma32(tb[i % KC], dsb[mb][i / DB], dk[i % DB]);
+          if constexpr (i + KC < NCS) {
+            if (WANT_DV) ta[i % KC] = tra.template read<Gt>(2 * mb + (i + KC) / DB, (i + KC) % DB);
+            if (WANT_DK) tb[i % KC] = tra.template read<Qt>(2 * mb + (i + KC) / DB, (i + KC) % DB);
+          }
+          pin_step();
+        });
+      });
+      return;
+    }
     phase_a(StageC<0>{});
     {
       constexpr int kAhead = NA < 6 ? NA : 6;
