@@ -167,7 +167,6 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a, const unsigned blo
   ktab.fill(ksum, reinterpret_cast<i32x4 *>(smem + L::kBytes), nt_all, tid, NT,
             [&](const tile_summary_t sm) { return sm.x <= qmax_g; });
   __syncthreads();
-  auto find = [&](int t) __attribute__((always_inline)) { return ktab.at(t).x; };
   const uint32_t smem0 = lds_addr(smem);
   // A tile is requested one load at a time (part p of LPT): the K loads, the V loads,
   // then the row of key ids.
@@ -271,8 +270,7 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a, const unsigned blo
       });
     });
   };
-  auto compute = [&](auto stage_c, int t, auto bg) __attribute__((always_inline)) {
-    const i32x4 e = ktab.at(t);
+  auto compute = [&](auto stage_c, const i32x4 e, auto bg) __attribute__((always_inline)) {
     const tile_summary_t sm = {e.y, e.z, e.w, 0};
     if (sm.x > qmax_w) return false;  // wave-uniform: no row of this wave sees a key of the tile
     if (sm.z != 0 && sm.y <= qmin_w)
@@ -284,7 +282,7 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a, const unsigned blo
 
   // Two LDS stages: while tile t is being used, tile t+1 streams into the other one.
   settle_loads();
-  tile_pipeline<NS, LPT, LPT>(0, nt, find, issue, compute);
+  tile_pipeline_tab<NS, LPT, LPT>(ktab, 0, nt, nt_all, issue, compute);
 
   // every wave is past its last tile (and its last request) before the tiles become output buffers
   __syncthreads();

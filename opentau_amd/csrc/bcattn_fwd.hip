@@ -185,7 +185,6 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
               [&](const tile_summary_t sm) { return sm.x <= qmax_g; });
     __syncthreads();
   }
-  auto find = [&](int t) __attribute__((always_inline)) { return ktab.at(t).x; };
   RowAddr<D> rowa;
   rowa.init(lane, smem0);
   TrAddr<D> tra;
@@ -351,12 +350,11 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
     wait_async_loads_but<0>();  // the early requests, if no row of the workgroup is valid
   } else {
     // While tile t is being used, the next needed tile(s) stream into the other stage(s).
-    auto compute = [&](auto stage_c, int t, auto bg) __attribute__((always_inline)) {
-      const i32x4 e = ktab.at(t);
+    auto compute = [&](auto stage_c, const i32x4 e, auto bg) __attribute__((always_inline)) {
       return compute_sm(stage_c, tile_summary_t{e.y, e.z, e.w, 0}, bg);
     };
     settle_loads();
-    tile_pipeline<NS, LPT, LPT>(t_first, nt, find, issue_part, compute);
+    tile_pipeline_tab<NS, LPT, LPT>(ktab, t_first, nt, nt_all, issue_part, compute);
   }
 
   // ---- epilogue ----------------------------------------------------------------

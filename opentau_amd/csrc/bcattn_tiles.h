@@ -428,6 +428,69 @@ __device__ __forceinline__ void tile_pipeline(int first, int end, Find find_at, 
   wait_async_loads_but<0>();  // the empty requests of the last steps
 }
 
+// The same walk for a kernel whose needed tiles come straight from one NeededTable (entry t = the first
+// needed tile at or after t, with its summary): the entry a step needs is read from LDS during the step
+// before and only moved to scalar registers where it is used, so neither the lookup of the next tile nor
+// the summary of the current one costs an LDS round trip on the way from one tile to the next.
+//   issue(t, StageC, StageC<part>, live)   as above
+//   compute(StageC, e, bg) -> bool         e = {tile, summary min, max, all valid} of the current tile
+// `end` is at most the table's tile count.
+template <int NS, int LPT, int NPARTS, class Issue, class Compute>
+__device__ __forceinline__ void tile_pipeline_tab(const NeededTable &tab, int first, int end, int ntab, Issue issue,
+                                                  Compute compute) {
+  static_assert(NS == 2 || NS == 3, "two or three stages");
+  auto clamp = [&](i32x4 e) {  // nothing needed in [t, end): tile index `end`
+    e.x = e.x < end ? e.x : end;
+    return e;
+  };
+  auto issue_all = [&](int t, auto sc, bool live) {
+    static_for<NPARTS>([&](auto part) { issue(t, sc, part, live); });
+  };
+  if (first >= end) return;
+  i32x4 e0 = clamp(tab.at(first));
+  if (e0.x >= end) return;
+  issue_all(e0.x, StageC<0>{}, true);
+  i32x4 e1 = clamp(tab.at(e0.x + 1 < ntab ? e0.x + 1 : ntab));
+  if (NS == 3) issue_all(e1.x < end ? e1.x : e0.x, StageC<1>{}, e1.x < end);
+  // the entry behind the newest known tile, on its way
+  auto ahead_of = [&](const i32x4 &e) { return tab.raw(e.x + 1 < ntab ? e.x + 1 : ntab); };
+  i32x4 raw = ahead_of(e1);
+  auto step = [&](auto sc) {
+    constexpr int S = decltype(sc)::value;
+    constexpr StageC<(S + NS - 1) % NS> into{};
+    i32x4 en;  // the tile due in this step, if any
+    if (NS == 2) {
+      en = e1;
+      wait_async_loads_but<0>();
+    } else {
+      en = clamp(uniform_summary(raw));
+      if (e1.x >= end) en.x = end;
+      raw = ahead_of(en);
+      wait_async_loads_but<LPT>();  // the newer tile stays in flight
+    }
+    tile_barrier();
+    const bool due = en.x < end;
+    const int tq = due ? en.x : e0.x;
+    if (!compute(sc, e0, [&](auto part) { issue(tq, into, part, due); })) issue_all(tq, into, due);
+    if (NS == 2) {
+      e0 = e1;
+      e1 = clamp(uniform_summary(raw));
+      if (e0.x >= end) e1.x = end;
+      raw = ahead_of(e1);
+    } else {
+      e0 = e1, e1 = en;
+    }
+    return e0.x >= end;
+  };
+  for (;;) {
+    if (step(StageC<0>{})) break;
+    if (step(StageC<1>{})) break;
+    if (NS == 3)
+      if (step(StageC<2>{})) break;
+  }
+  wait_async_loads_but<0>();  // the empty requests of the last steps
+}
+
 // Short tile ranges (a split of the key axis): the tiles [first, end) are taken in
 // order, none is skipped, and as many as there are LDS stages are requested at once,
 // so that a range of at most NS tiles pays the memory latency once.  The caller has
