@@ -401,15 +401,6 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, const unsigned bl
   gld.init(tid, a.d_o.ss);
   const uint32_t qstep = (uint32_t)(64 * a.q.ss * 2), gstep = (uint32_t)(64 * a.d_o.ss * 2);
 
-  // first needed iteration at or after `it`: in its head, else the first of the next head
-  // (every head has the same needed tiles)
-  auto find = [&](int it) __attribute__((always_inline)) {
-    const int g = it >> 16, qt = it & 0xffff;
-    const int nn = qtab.at(qt < nqt ? qt : nqt).x;
-    if (nn < nqt) return (g << 16) | nn;
-    const int first = qtab.at(0).x;
-    return first < nqt ? ((g + 1) << 16) | first : nit;
-  };
   const uint32_t smem0 = lds_addr(smem);
   // A tile is requested one load at a time (part p of LPT): the Q loads, the dO loads,
   // then the wave's statistics row.  Part 0 works out where the tile is.
@@ -653,8 +644,7 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, const unsigned bl
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-  auto compute = [&](auto stage_c, int it, auto bg) __attribute__((always_inline)) {
-    const i32x4 e = qtab.at(it & 0xffff);
+  auto compute = [&](auto stage_c, const i32x4 e, auto bg) __attribute__((always_inline)) {
     const tile_summary_t sm = {e.y, e.z, e.w, 0};
     if (sm.y < kmin_w) return false;  // wave-uniform: no key of this wave is seen by the tile
     if (sm.z != 0 && allk_w != 0 && kmax_w <= sm.x)
@@ -665,7 +655,7 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, const unsigned bl
   };
 
   settle_loads();
-  tile_pipeline<NS, LPT, LPT>(it0, nit, find, issue, compute);
+  tile_pipeline_heads<NS, LPT, LPT>(qtab, it0, nit, nqt, issue, compute);
 
   if (jok && HS > 1) {
     // this workgroup's share of the sums, fp32, for bwd_dkv_reduce_kernel

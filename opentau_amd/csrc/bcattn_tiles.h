@@ -491,6 +491,70 @@ __device__ __forceinline__ void tile_pipeline_tab(const NeededTable &tab, int fi
   wait_async_loads_but<0>();  // the empty requests of the last steps
 }
 
+// And for the dK/dV kernels, whose iterations run over (query head, needed query tile), head-major, as
+// head << 16 | tile: every head has the same needed tiles, so the iteration after (g, t) is (g, the first
+// needed tile after t) or, when there is none, (g + 1, the first needed tile at all).  Iterations
+// [first, end), both of the form head << 16; `ntab` tiles in the table.
+//   compute(StageC, e, bg) -> bool         e = {head << 16 | tile, summary min, max, all valid}
+template <int NS, int LPT, int NPARTS, class Issue, class Compute>
+__device__ __forceinline__ void tile_pipeline_heads(const NeededTable &tab, int first, int end, int ntab, Issue issue,
+                                                    Compute compute) {
+  static_assert(NS == 2 || NS == 3, "two or three stages");
+  auto issue_all = [&](int it, auto sc, bool live) {
+    static_for<NPARTS>([&](auto part) { issue(it, sc, part, live); });
+  };
+  if (first >= end) return;
+  const i32x4 e_first = tab.at(0);  // first needed tile of a head
+  if (e_first.x >= ntab) return;
+  // the iteration after `cur`, given the table entry behind cur's tile
+  auto after = [&](const i32x4 &cur, i32x4 e) {
+    int g = cur.x >> 16;
+    if (e.x >= ntab) e = e_first, g += 1;
+    const int it = (g << 16) | e.x;
+    e.x = cur.x < end && it < end ? it : end;
+    return e;
+  };
+  auto ahead_of = [&](const i32x4 &e) { return tab.raw((e.x & 0xffff) + 1 < ntab ? (e.x & 0xffff) + 1 : ntab); };
+  i32x4 e0 = e_first;
+  e0.x |= first;
+  issue_all(e0.x, StageC<0>{}, true);
+  i32x4 e1 = after(e0, uniform_summary(ahead_of(e0)));
+  if (NS == 3) issue_all(e1.x < end ? e1.x : e0.x, StageC<1>{}, e1.x < end);
+  i32x4 raw = ahead_of(e1);
+  auto step = [&](auto sc) {
+    constexpr int S = decltype(sc)::value;
+    constexpr StageC<(S + NS - 1) % NS> into{};
+    i32x4 en;  // the iteration due in this step, if any
+    if (NS == 2) {
+      en = e1;
+      wait_async_loads_but<0>();
+    } else {
+      en = after(e1, uniform_summary(raw));
+      raw = ahead_of(en);
+      wait_async_loads_but<LPT>();  // the newer tile stays in flight
+    }
+    tile_barrier();
+    const bool due = en.x < end;
+    const int tq = due ? en.x : e0.x;
+    if (!compute(sc, e0, [&](auto part) { issue(tq, into, part, due); })) issue_all(tq, into, due);
+    if (NS == 2) {
+      e0 = e1;
+      e1 = after(e0, uniform_summary(raw));
+      raw = ahead_of(e1);
+    } else {
+      e0 = e1, e1 = en;
+    }
+    return e0.x >= end;
+  };
+  for (;;) {
+    if (step(StageC<0>{})) break;
+    if (step(StageC<1>{})) break;
+    if (NS == 3)
+      if (step(StageC<2>{})) break;
+  }
+  wait_async_loads_but<0>();  // the empty requests of the last steps
+}
+
 // Short tile ranges (a split of the key axis): the tiles [first, end) are taken in
 // order, none is skipped, and as many as there are LDS stages are requested at once,
 // so that a range of at most NS tiles pays the memory latency once.  The caller has
