@@ -161,10 +161,35 @@ def main() -> int:
             result["dispatch"] = {n: bench_dispatch(torch, fa, workload(n), dev) for n in ("c3", "c5")}
             result["reference_harness"] = bench_reference_harness(torch, fa, dev)
             result["rope"] = bench_rope(torch, dev)
+            result["matrix_ceiling"] = matrix_ceiling(result["value"], result["roofline"])
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, workload(args.workload))
     print(json.dumps(result))
     return 0
+
+
+def matrix_ceiling(step_tflops, roofline):
+    """What this GPU's matrix pipes sustain, measured beside the step: ``opentau_amd/csrc/probe/mfma_ceiling``
+    (its own process; a loop of the bf16 MFMA the kernels use with one LDS operand read per product, two waves
+    per SIMD, nothing else) with constant operands and with operands of pseudo-random sign and mantissa.  The
+    second is the rate real data can reach under the chip's power management; the published peak that
+    ``roofline.peak`` must quote is computed at the nominal clock.  The step *executes* 18 product units for
+    the 14 it is credited with (S and dP are formed in both backward kernels), the dominant kernel 8 for 6."""
+    import subprocess
+
+    exe = ROOT / "opentau_amd" / "csrc" / "probe" / "mfma_ceiling"
+    if not exe.exists():
+        return None
+    try:
+        out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120, check=True).stdout
+        rec = json.loads(out.strip().splitlines()[-1])
+    except (subprocess.SubprocessError, ValueError, IndexError) as e:
+        return {"error": str(e)[:200]}
+    sustained = rec["tflops_random_operands"]
+    rec["step_credited_frac_of_sustained"] = round(step_tflops / sustained, 4)
+    rec["step_executed_frac_of_sustained"] = round(step_tflops * 18 / 14 / sustained, 4)
+    rec["dominant_kernel_executed_frac_of_sustained"] = round(roofline["achieved"] * 8 / 6 / sustained, 4)
+    return rec
 
 
 def bench_train(torch, fa, w, dev, steps, warmup):

@@ -1,0 +1,90 @@
+// What the matrix pipes of this GPU sustain, measured: a loop of v_mfma_f32_32x32x16_bf16 with one
+// 16-byte-per-lane LDS operand read per product (the operand pattern of the attention kernels: one
+// operand in registers, one read from the tile in LDS), two waves per SIMD on every CU, nothing else.
+// Run once with constant operands and once with operands of pseudo-random sign and mantissa: the
+// second draws more power and the clock settles lower, so it is the rate that real data can reach.
+// Prints one JSON line.  A measurement aid: the library does not use it.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define CHECK(x)                                                                   \
+  do {                                                                             \
+    hipError_t e_ = (x);                                                           \
+    if (e_ != hipSuccess) {                                                        \
+      fprintf(stderr, "%s: %s\n", #x, hipGetErrorString(e_));                      \
+      exit(1);                                                                     \
+    }                                                                              \
+  } while (0)
+
+// Four independent accumulators per wave; each product's LDS operand is re-read right after the
+// product that used it, three products before its next use (lgkmcnt(3) is the wait for that).
+__global__ __launch_bounds__(512) void mfma_lds_loop(float *out, int iters, int random_data) {
+  __shared__ __align__(16) char tile[65536];
+  for (int i = threadIdx.x; i < 65536 / 4; i += 512) {
+    unsigned h = (i * 2654435761u) ^ ((i >> 3) * 40503u);
+    // two bf16 per word: exponent of [0.5, 1), sign and mantissa from the hash (or 1.0, 1.0)
+    reinterpret_cast<unsigned *>(tile)[i] = random_data ? ((h & 0x807f807fu) | 0x3f003f00u) : 0x3f803f80u;
+  }
+  __syncthreads();
+  bf16x8 b, r[4];
+  for (int e = 0; e < 8; ++e)
+    b[e] = random_data ? (__bf16)((float)((int)((threadIdx.x * 37 + e * 11) % 17) - 8) * 0.013f) : (__bf16)(e * 0.5f);
+  f32x16 acc[4];
+  for (int i = 0; i < 4; ++i) {
+    for (int x = 0; x < 16; ++x) acc[i][x] = 0.f;
+    for (int e = 0; e < 8; ++e) r[i][e] = (__bf16)1.0f;
+  }
+  const unsigned addr = (unsigned)(size_t)tile + (threadIdx.x & 63) * 16 + (threadIdx.x >> 6) * 4096;
+  for (int it = 0; it < iters; ++it) {
+    asm volatile("s_waitcnt lgkmcnt(3)\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\tds_read_b128 %1, %3"
+                 : "+v"(acc[0]), "+v"(r[0]) : "v"(b), "v"(addr));
+    asm volatile("s_waitcnt lgkmcnt(3)\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\tds_read_b128 %1, %3 offset:1024"
+                 : "+v"(acc[1]), "+v"(r[1]) : "v"(b), "v"(addr));
+    asm volatile("s_waitcnt lgkmcnt(3)\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\tds_read_b128 %1, %3 offset:2048"
+                 : "+v"(acc[2]), "+v"(r[2]) : "v"(b), "v"(addr));
+    asm volatile("s_waitcnt lgkmcnt(3)\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\tds_read_b128 %1, %3 offset:3072"
+                 : "+v"(acc[3]), "+v"(r[3]) : "v"(b), "v"(addr));
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  float s = 0.f;
+  for (int i = 0; i < 4; ++i)
+    for (int x = 0; x < 16; ++x) s += acc[i][x];
+  out[blockIdx.x * 512 + threadIdx.x] = s;
+}
+
+int main() {
+  hipDeviceProp_t prop;
+  CHECK(hipGetDeviceProperties(&prop, 0));
+  const int cus = prop.multiProcessorCount;
+  float *out;
+  CHECK(hipMalloc(&out, (size_t)cus * 512 * sizeof(float)));
+  hipEvent_t e0, e1;
+  CHECK(hipEventCreate(&e0));
+  CHECK(hipEventCreate(&e1));
+  const int iters = 200000, reps = 12;  // 0.8 M products per wave and launch: 20-30 ms
+  double rate[2] = {0, 0};
+  for (int kind = 0; kind < 2; ++kind) {
+    float sum = 0.f;
+    for (int rep = 0; rep < reps; ++rep) {
+      CHECK(hipEventRecord(e0));
+      hipLaunchKernelGGL(mfma_lds_loop, dim3(cus), dim3(512), 0, 0, out, iters, kind);
+      CHECK(hipEventRecord(e1));
+      CHECK(hipEventSynchronize(e1));
+      float ms;
+      CHECK(hipEventElapsedTime(&ms, e0, e1));
+      if (rep >= reps / 2) sum += ms;  // the second half of the launches: the clock has settled
+    }
+    const double flop = (double)cus * 8 * 4 * iters * 32768.0;
+    rate[kind] = flop / (sum / (reps - reps / 2) * 1e-3) / 1e12;
+  }
+  printf("{\"kernel\": \"v_mfma_f32_32x32x16_bf16 + one ds_read_b128 per product, 2 waves/SIMD\", \"cus\": %d, "
+         "\"tflops_constant_operands\": %.0f, \"tflops_random_operands\": %.0f}\n",
+         cus, rate[0], rate[1]);
+  CHECK(hipFree(out));
+  return 0;
+}
