@@ -532,22 +532,28 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, const unsigned bl
       // operand reads KA / KC products ahead; those are written out as rings of registers and pinned
       // step by step (left to the scheduler, the reads of the dK form end up one product ahead, each
       // product waiting out a whole LDS round trip).
+      // A ring's first reads go out during the last steps of the phase before it (the accumulating
+      // ring's before the softmax, the second half's row ring under the first half's accumulating
+      // products), so only the first ring of a tile, right behind the tile barrier, waits out an LDS
+      // round trip with nothing else to do.
       Stats st;
+      constexpr int KA = 3, KC = 4, NCS = 2 * DB;
+      e16x8 fq[KA], fg[WANT_DK ? KA : 1];
+#pragma unroll
+      for (int i = 0; i < KA; ++i) {
+        fq[i] = rowa.template read<Qt>(0, i);
+        if (WANT_DK) fg[i] = rowa.template read<Gt>(0, i);
+      }
       static_for<2>([&](auto mb_c) {
         constexpr int mb = decltype(mb_c)::value;
-        constexpr int KA = 3, KC = 4;
         load_stats(mb, st);
-        e16x8 fq[KA], fg[WANT_DK ? KA : 1];
-#pragma unroll
-        for (int i = 0; i < KA; ++i) {
-          fq[i] = rowa.template read<Qt>(32 * mb, i);
-          if (WANT_DK) fg[i] = rowa.template read<Gt>(32 * mb, i);
-        }
 #pragma unroll
         for (int x = 0; x < 16; ++x) {
           s[mb][x] = 0.f;
           if constexpr (WANT_DK) dp[mb][x] = 0.f;
         }
+        // accumulating products: step i is (16-query quarter i / DB of the half, head_dim block i % DB)
+        e16x8 ta[WANT_DV ? KC : 1], tb[WANT_DK ? KC : 1];
         pin_step();
         static_for<DK>([&](auto ks_c) {
           constexpr int ks = decltype(ks_c)::value;
@@ -558,18 +564,14 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, const unsigned bl
             fq[ks % KA] = rowa.template read<Qt>(32 * mb, ks + KA);
             if (WANT_DK) fg[ks % KA] = rowa.template read<Gt>(32 * mb, ks + KA);
           }
+          if constexpr (ks >= DK - KC) {
+            constexpr int j = ks - (DK - KC);
+            if (WANT_DV) ta[j] = tra.template read<Gt>(2 * mb + j / DB, j % DB);
+            if (WANT_DK) tb[j] = tra.template read<Qt>(2 * mb + j / DB, j % DB);
+          }
           pin_step();
         });
         softmax(mb, st);
-        pin_step();
-        // accumulating products: step i is (16-query quarter i / DB of the half, head_dim block i % DB)
-        constexpr int NCS = 2 * DB;
-        e16x8 ta[WANT_DV ? KC : 1], tb[WANT_DK ? KC : 1];
-#pragma unroll
-        for (int i = 0; i < KC; ++i) {
-          if (WANT_DV) ta[i] = tra.template read<Gt>(2 * mb + i / DB, i % DB);
-          if (WANT_DK) tb[i] = tra.template read<Qt>(2 * mb + i / DB, i % DB);
-        }
         pin_step();
         static_for<NCS>([&](auto i_c) {
           constexpr int i = decltype(i_c)::value;
@@ -578,6 +580,11 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, const unsigned bl
           if constexpr (i + KC < NCS) {
             if (WANT_DV) ta[i % KC] = tra.template read<Gt>(2 * mb + (i + KC) / DB, (i + KC) % DB);
             if (WANT_DK) tb[i % KC] = tra.template read<Qt>(2 * mb + (i + KC) / DB, (i + KC) % DB);
+          }
+          if constexpr (mb == 0 && i >= NCS - KA) {
+            constexpr int j = i - (NCS - KA);
+            fq[j] = rowa.template read<Qt>(32, j);
+            if (WANT_DK) fg[j] = rowa.template read<Gt>(32, j);
           }
           pin_step();
         });
