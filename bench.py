@@ -14,7 +14,10 @@ the launch stream, which gives the per-kernel durations behind ``roofline``.
 the outputs) beside the raw C-ABI step; ``denoise`` the pi0.5 inference attention
 (18 prefix calls + 180 cached-suffix calls at B=8) and pi0.6's (34 x 5 suffix
 calls at B=16); ``cpu_baseline`` is the eager CPU oracle on a bounded slice of
-the headline workload, in the workload's own dtype.
+the headline workload, in the workload's own dtype; ``matrix_ceiling`` is what a
+bare MFMA loop sustains on this GPU (measured in the same run) and ``torch_sdpa``
+the reference's ``sdpa`` call through PyTorch-ROCm on the same tensors (both
+informational).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-denoise]
 """
@@ -162,6 +165,9 @@ def main() -> int:
             result["reference_harness"] = bench_reference_harness(torch, fa, dev)
             result["rope"] = bench_rope(torch, dev)
             result["matrix_ceiling"] = matrix_ceiling(result["value"], result["roofline"])
+            result["torch_sdpa"] = {n: bench_torch_sdpa(torch, workload(n), dev,
+                                                        result["ms_per_step"] if n == "c5" else others[n]["ms_per_step"])
+                                    for n in ("c3", "c5")}
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, workload(args.workload))
     print(json.dumps(result))
@@ -281,6 +287,51 @@ def bench_train(torch, fa, w, dev, steps, warmup):
         "flops_per_step": 14 * unit,
         "roofline": roofline,
     }
+
+
+def bench_torch_sdpa(torch, w, dev, our_ms, iters=5, warmup=2):
+    """Informational: what the reference's ``sdpa`` attention costs on this GPU through PyTorch-ROCm, on
+    the same tensors.  The call is the reference's (``pi05/paligemma_with_expert.py:955-1035``): K and V
+    expanded to all query heads, ``(B,H,S,D)`` views, a dense boolean ``(B,1,S,S)`` mask (built once, outside
+    the timed region), ``scaled_dot_product_attention`` without ``is_causal``; forward + backward by
+    autograd, HIP-event median.  Whatever kernel PyTorch picks for a masked call is what runs."""
+    import torch.nn.functional as F
+
+    q_blk, k_blk, q_valid, k_valid = (t.to(dev) for t in w.block_ids())
+    mask = (q_valid[:, :, None] & k_valid[:, None, :] & (k_blk[:, None, :] <= q_blk[:, :, None]))[:, None]
+    q, k, v = (t.to(dev).requires_grad_(True) for t in (w.q, w.k, w.v))
+    go = w.d_out.to(dev)
+    grp = w.H // w.Hkv
+
+    def step():
+        kx = k[:, :, :, None, :].expand(w.B, w.S, w.Hkv, grp, w.D).reshape(w.B, w.S, w.H, w.D)
+        vx = v[:, :, :, None, :].expand(w.B, w.S, w.Hkv, grp, w.D).reshape(w.B, w.S, w.H, w.D)
+        o = F.scaled_dot_product_attention(q.transpose(1, 2), kx.transpose(1, 2), vx.transpose(1, 2),
+                                           attn_mask=mask, dropout_p=0.0, is_causal=False, scale=w.scale)
+        o.transpose(1, 2).backward(go)
+        q.grad = k.grad = v.grad = None
+
+    torch.cuda.reset_peak_memory_stats(dev)
+    try:
+        for _ in range(warmup):
+            step()
+        ms = []
+        for _ in range(iters):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            step()
+            e1.record()
+            torch.cuda.synchronize()
+            ms.append(e0.elapsed_time(e1))
+    except RuntimeError as exc:
+        return {"error": str(exc)[:200]}
+    finally:
+        del mask
+        torch.cuda.empty_cache()
+    med = statistics.median(ms)
+    return {"workload": f"{w.name}: B{w.B} H{w.H} Hkv{w.Hkv} D{w.D} S{w.S}", "fwd_bwd_ms": round(med, 3),
+            "peak_memory_gb": round(torch.cuda.max_memory_allocated(dev) / 2**30, 2),
+            "this_library_ms": our_ms, "ratio": round(med / our_ms, 2)}
 
 
 def bench_dispatch(torch, fa, w, dev, steps=20, warmup=3):
