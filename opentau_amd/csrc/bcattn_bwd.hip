@@ -65,13 +65,6 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const BwdArgs a) {
 }
 
 // LDS stages: three where they fit in the 160 KB of a CU, else two.
-// Ends a step of a hand-ordered sequence: neither the compiler's code motion (the empty asm statement with
-// its memory clobber holds the LDS reads in place) nor the instruction scheduler moves anything across.
-__device__ __forceinline__ void pin_step() {
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_sched_barrier(0);
-}
-
 template <int D>
 struct BwdStages {
   static constexpr int value = D <= 128 ? 3 : 2;

@@ -33,6 +33,10 @@ struct SplitStages {
 
 // TWOSEG: the keys come as two segments (cache, then new); with one segment the tile requests
 // choose nothing at run time.
+#ifndef BCATTN_FWD_INTERLEAVED
+#define BCATTN_FWD_INTERLEAVED 1
+#endif
+
 template <int D, int NW, bool SPLIT, bool TWOSEG>
 __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, const SplitArgs sp) {
   using T = Tile<D>;
@@ -201,8 +205,159 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
   float l = 0.f;        // this lane half's share of the running sum
   const float c = a.scale * kLog2e;
 
+  // head_dim 256: one wave per SIMD, so only this wave's own products can run beside its softmax
+  // arithmetic, and only if the program says so instruction by instruction.  The tile goes as two
+  // 32-key halves: [S of half 0] [S of half 1 beside the softmax of half 0] [P V of half 0 beside the
+  // softmax of half 1] [P V of half 1].  Operand reads run through rings of registers that carry on
+  // from one phase into the next; every step (one product, its read, its share of the arithmetic) is
+  // closed by pin_step(), the products and the arithmetic are tied to their step by empty asm
+  // statements (without them instruction selection sinks them behind the last product).
+  // The running reference follows the half's maximum only when that has outgrown it by 2^8; O and the
+  // row sum are then rescaled between two phases (O is being accumulated into during the phase in
+  // which the second half's maximum is found).
+  auto compute_il = [&](auto stage_c, auto masked_c, auto bg) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_c)::value != 0;
+    constexpr int S = decltype(stage_c)::value;
+    constexpr int Kt = L::tile(S, 0), Vt = L::tile(S, 1);
+    const int *kb_s = reinterpret_cast<const int *>(smem + L::aux(S));
+    constexpr int KA = 3, KC = 4;
+    constexpr int NPV = 2 * DB;  // P V products of a half: (16-key quarter, 32-row block of O^T)
+    f32x16 s[2];
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int x = 0; x < 16; ++x) s[mb][x] = 0.f;
+    e16x8 fk[KA], tv[KC], pb[4];
+#pragma unroll
+    for (int i = 0; i < KA; ++i) fk[i] = rowa.template read<Kt>(0, i);
+    pin_step();
+    // the next row read of the ring: the rows of half 0, then those of half 1
+    auto next_rows = [&](auto nx_c) __attribute__((always_inline)) {
+      constexpr int nx = decltype(nx_c)::value;
+      if constexpr (nx < DK)
+        fk[nx % KA] = rowa.template read<Kt>(0, nx);
+      else if constexpr (nx < 2 * DK)
+        fk[nx % KA] = rowa.template read<Kt>(32, nx - DK);
+    };
+    // the next transposing read: product nx of the 2 * NPV of the tile
+    auto next_cols = [&](auto nx_c) __attribute__((always_inline)) {
+      constexpr int nx = decltype(nx_c)::value;
+      if constexpr (nx < 2 * NPV) tv[nx % KC] = tra.template read<Vt>(nx / DB, nx % DB);
+    };
+    // ---- the softmax of one half, in the pieces that the steps of a phase take --------------
+    float mloc = 0.f, lt = 0.f, corr = 1.f, sv[16];  // sv: the half's scores, then its exponentials
+    i32x4 kb4[4];
+    bool grown = false;
+    // piece J of half H (J = 0 .. 15)
+    auto softmax_piece = [&](auto h_c, auto j_c) __attribute__((always_inline)) {
+      constexpr int H = decltype(h_c)::value, J = decltype(j_c)::value;
+      if constexpr (J == 0) {
+        if constexpr (MASKED) {
+#pragma unroll
+          for (int r4 = 0; r4 < 4; ++r4) kb4[r4] = *reinterpret_cast<const i32x4 *>(kb_s + 32 * H + 8 * r4 + 4 * hh);
+        }
+      } else if constexpr (J <= 4) {  // out of the accumulator: mask and maximum of elements 4 (J-1) .. +3
+        constexpr int r4 = J - 1;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          const int e = 4 * r4 + x;
+          sv[e] = (MASKED && kb4[r4][x] > qb) ? -INFINITY : s[H][e];
+          mloc = e == 0 ? sv[0] : fmaxf(mloc, sv[e]);
+        }
+        asm volatile("" : "+v"(mloc), "+v"(sv[4 * r4]), "+v"(sv[4 * r4 + 1]), "+v"(sv[4 * r4 + 2]), "+v"(sv[4 * r4 + 3]));
+      } else if constexpr (J == 5) {  // the row's maximum over the half; does the reference move?
+        mloc = fmaxf(mloc, swap32(mloc));
+        const bool grow = (mloc - m) * c > 8.f;  // false for a fully masked half (mloc = -inf)
+        const float mnew = grow ? mloc : m;
+        const float moff_new = (mnew == -INFINITY) ? 0.f : mnew * c;
+        // 1 where the reference stays; a row without one has accumulated nothing that counts
+        corr = !grow ? 1.f : (m == -INFINITY) ? 0.f : fast_exp2(moff - moff_new);
+        grown = __any(grow);
+        m = mnew;
+        moff = moff_new;
+        lt = 0.f;
+        asm volatile("" : "+v"(corr), "+v"(moff), "+v"(m));
+      } else if constexpr (J <= 13) {  // two exponentials
+        constexpr int e = 2 * (J - 6);
+        sv[e] = fast_exp2(sv[e] * c - moff);
+        sv[e + 1] = fast_exp2(sv[e + 1] * c - moff);
+        lt += sv[e] + sv[e + 1];
+        asm volatile("" : "+v"(sv[e]), "+v"(sv[e + 1]), "+v"(lt));
+      } else {  // eight of them to 16 bits
+        constexpr int q = J - 14;
+        pb[2 * H + q] = pack8(sv[8 * q], sv[8 * q + 1], sv[8 * q + 2], sv[8 * q + 3], sv[8 * q + 4], sv[8 * q + 5],
+                              sv[8 * q + 6], sv[8 * q + 7]);
+        asm volatile("" : "+v"(pb[2 * H + q]));
+      }
+    };
+    auto rescale = [&]() __attribute__((always_inline)) {
+      if (grown) {
+        // (O lives in accumulation registers; it is tied to them on both sides of this rare block, or the
+        // compiler keeps it in vector registers around the block and moves all of it on every tile)
+#pragma unroll
+        for (int db = 0; db < DB; ++db) asm volatile("" : "+a"(o[db]));
+        l *= corr;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int x = 0; x < 16; ++x) o[db][x] *= corr;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) asm volatile("" : "+a"(o[db]));
+      }
+      l += lt;
+    };
+    // ---- A: S of keys 0..31 ------------------------------------------------------------------
+    static_for<DK>([&](auto ks_c) {
+      constexpr int ks = decltype(ks_c)::value;
+      parts_at_slot<ks, DK, LPT>(bg);  // (all requests in this phase: no vector arithmetic competes for issue)
+      s[0] = mfma32(fk[ks % KA], qf[ks], s[0]);
+      asm volatile("" : "+a"(s[0]));
+      next_rows(StageC<ks + KA>{});
+      pin_step();
+    });
+    // ---- B: S of keys 32..63 beside the softmax of half 0 --------------------------------------
+    static_for<DK>([&](auto ks_c) {
+      constexpr int ks = decltype(ks_c)::value;
+      s[1] = mfma32(fk[(DK + ks) % KA], qf[ks], s[1]);
+      asm volatile("" : "+a"(s[1]));
+      next_rows(StageC<DK + ks + KA>{});
+      if constexpr (ks >= DK - KC) next_cols(StageC<ks - (DK - KC)>{});
+      softmax_piece(StageC<0>{}, ks_c);
+      pin_step();
+    });
+    rescale();  // (P V of the tile before has long been issued; nothing accumulates into O in phase B)
+    pin_step();
+    // ---- C: P V of half 0 beside the softmax of half 1 -----------------------------------------
+    static_for<NPV>([&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      o[i % DB] = mfma32(tv[i % KC], pb[i / DB], o[i % DB]);
+      asm volatile("" : "+a"(o[i % DB]));
+      next_cols(StageC<i + KC>{});
+      softmax_piece(StageC<1>{}, i_c);
+      pin_step();
+    });
+    rescale();
+    pin_step();
+    // ---- D: P V of half 1 ------------------------------------------------------------------------
+    static_for<NPV>([&](auto i_c) {
+      constexpr int i = NPV + decltype(i_c)::value;
+      o[i % DB] = mfma32(tv[i % KC], pb[i / DB], o[i % DB]);
+      asm volatile("" : "+a"(o[i % DB]));
+      next_cols(StageC<i + KC>{});
+      pin_step();
+    });
+  };
+
   auto compute_sm = [&](auto stage_c, const tile_summary_t sm, auto bg) __attribute__((always_inline)) {
     if (sm.x > qmax_w) return false;  // wave-uniform: no row of this wave sees a key of the tile
+    if constexpr (BCATTN_FWD_INTERLEAVED && D == 256) {
+      static_assert(DK == 2 * DB && DK == 16, "the phases are written for 16 steps each");
+      if (!(sm.z != 0 && sm.y <= qmin_w))
+        compute_il(stage_c, StageC<1>{}, bg);
+      else  // every row of the wave sees every key of the tile
+        compute_il(stage_c, StageC<0>{}, bg);
+      return true;
+    }
     constexpr int S = decltype(stage_c)::value;
     constexpr int Kt = L::tile(S, 0), Vt = L::tile(S, 1);
     const int *kb_s = reinterpret_cast<const int *>(smem + L::aux(S));

@@ -354,6 +354,13 @@ __device__ __forceinline__ void wait_async_loads_but() {
 // the loads that are meant to stay in flight.
 __device__ __forceinline__ void tile_barrier() { asm volatile("s_barrier" ::: "memory"); }
 
+// Ends a step of a hand-ordered sequence: neither the compiler's code motion (the empty asm statement with
+// its memory clobber holds the LDS reads in place) nor the instruction scheduler moves anything across.
+__device__ __forceinline__ void pin_step() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+}
+
 // Spreads `PARTS` requests over `SLOTS` places in order: at slot S, calls bg(StageC<p>{})
 // for every part p that belongs there (part p sits at slot p*SLOTS/PARTS).
 template <int S, int SLOTS, int PARTS, class Bg>
