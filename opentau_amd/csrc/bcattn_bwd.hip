@@ -1019,33 +1019,64 @@ __device__ __forceinline__ void bwd_dkv_pair_body(const BwdArgs &a, const unsign
         for (int x = 0; x < 4; ++x) dp[4 * r4 + x] = nd4[x];
       }
     }
-    if constexpr (CUR)
+    if constexpr (CUR) {
+      // Written out in issue order: per product of the chain its row read KA products ahead and its
+      // share of the dS arithmetic (one or two pairs of elements: 16-bit P to fp32, times dP - delta,
+      // the pair back to 16 bits), each step closed by pin_step().  The arithmetic starts at the third
+      // product: P was written just before the barrier and its read has to come back first.  (Left to
+      // schedule groups, the half step that also issues the tile requests had all of the arithmetic
+      // behind the chain, between the two groups of products of the wave that the other one waits for.)
+      constexpr int KA = DK < 4 ? DK : 4;
+      e16x8 fr[KA], pbx[2];
+      i32x4 wds[2];
+#pragma unroll
+      for (int i = 0; i < KA; ++i) fr[i] = rowa.template read<Gt>(32 * mb, i);
+      if constexpr (PREV) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) pbx[half] = lds_e16x8(x_lane + (1 - xcur) * XBYTES + half * 1024);
+      }
+      pin_step();
+      auto ds_pair = [&](auto q_c) __attribute__((always_inline)) {
+        constexpr int q = decltype(q_c)::value, half = q / 4, j = q % 4;
+        typedef e16_t e16x2_t __attribute__((ext_vector_type(2)));
+        e16x2_t r;
+        r[0] = (e16_t)((float)pbx[half][2 * j] * dp_prev[8 * half + 2 * j]);  // dp_prev = dP - delta
+        r[1] = (e16_t)((float)pbx[half][2 * j + 1] * dp_prev[8 * half + 2 * j + 1]);
+        wds[half][j] = __builtin_bit_cast(int, r);
+        asm volatile("" : "+v"(wds[half][j]));
+      };
       static_for<DK>([&](auto i_c) {
         constexpr int i = decltype(i_c)::value;
         parts_at_slot<i, DK, LPT>(bg);
-        dp = mfma32(rowa.template read<Gt>(32 * mb, i), frag[i], dp);
+        dp = mfma32(fr[i % KA], frag[i], dp);
+        asm volatile("" : "+v"(dp));
+        if constexpr (i + KA < DK) fr[i % KA] = rowa.template read<Gt>(32 * mb, i + KA);
+        if constexpr (PREV && DK == 8) {
+          if constexpr (i == 2 || i == 3) {
+            ds_pair(StageC<2 * (i - 2)>{});
+            ds_pair(StageC<2 * (i - 2) + 1>{});
+          } else if constexpr (i >= 4) {
+            ds_pair(StageC<i>{});
+          }
+        }
+        pin_step();
       });
-    else
-      static_for<LPT>([&](auto part) { bg(part); });
-    if constexpr (PREV) {
-#pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        const e16x8 pb = lds_e16x8(x_lane + (1 - xcur) * XBYTES + half * 1024);
-        float ds[8];
-#pragma unroll
-        for (int x = 0; x < 8; ++x) ds[x] = (float)pb[x] * dp_prev[8 * half + x];  // dp_prev = dP - delta
-        dsb[half] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
+      if constexpr (PREV) {
+        if constexpr (DK != 8) static_for<8>([&](auto q_c) { ds_pair(q_c); });
+        dsb[0] = __builtin_bit_cast(e16x8, wds[0]);
+        dsb[1] = __builtin_bit_cast(e16x8, wds[1]);
       }
-    }
-    if constexpr (CUR) {
-      // per product of dP: its row read and a share of the dS arithmetic
-      constexpr int VA = PREV ? (3 * 16 + DK - 1) / DK : 0;
-      __builtin_amdgcn_sched_group_barrier(0x100, (PREV ? 6 : 0) + 4, 0);
+    } else {
+      static_for<LPT>([&](auto part) { bg(part); });
+      if constexpr (PREV) {
 #pragma unroll
-      for (int x = 0; x < DK; ++x) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        if (VA) __builtin_amdgcn_sched_group_barrier(0x002, VA, 0);
+        for (int half = 0; half < 2; ++half) {
+          const e16x8 pb = lds_e16x8(x_lane + (1 - xcur) * XBYTES + half * 1024);
+          float ds[8];
+#pragma unroll
+          for (int x = 0; x < 8; ++x) ds[x] = (float)pb[x] * dp_prev[8 * half + x];  // dp_prev = dP - delta
+          dsb[half] = pack8(ds[0], ds[1], ds[2], ds[3], ds[4], ds[5], ds[6], ds[7]);
+        }
       }
     }
     __builtin_amdgcn_sched_barrier(0);
