@@ -29,38 +29,58 @@ namespace bcattn {
 inline namespace BCATTN_ELEM_NS {
 
 // ---- prep: delta and scaled LSE, padded -------------------------------------------
+// One row (b, h, i) per D/8 lanes, kPrepRows rows per thread with all of their loads in flight
+// together.  Rows are taken in the order in which they lie in memory: heads fastest where a token's
+// heads are neighbours ((B,S,H,D) tensors), tokens fastest otherwise.
+constexpr int kPrepRows = 4;
 template <int D>
 __global__ __launch_bounds__(256) void bwd_prep_kernel(const BwdArgs a) {
   constexpr int LPR = D / 8;
   constexpr int RPB = 256 / LPR;
-  const int Sqp = a.Sq_pad;
-  const int64_t total = (int64_t)a.B * a.H * Sqp;  // (b, h, i) with i fastest
-  const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
+  const uint32_t Sqp = (uint32_t)a.Sq_pad, H = (uint32_t)a.H;
+  const uint32_t total = (uint32_t)a.B * H * Sqp;  // (the launcher checks that this fits)
+  const bool hfast = a.o.sh < a.o.ss;
+  const uint32_t row0 = blockIdx.x * (uint32_t)(RPB * kPrepRows) + threadIdx.x / LPR;
   const int c = threadIdx.x % LPR;
-  float acc = 0.f;
-  int h = 0, i = 0, b = 0;
-  bool real = false;
-  if (row < total) {
-    i = (int)(row % Sqp);
-    h = (int)((row / Sqp) % a.H);
-    b = (int)(row / ((int64_t)Sqp * a.H));
-    real = i < a.Sq;
-    if (real) {
-      const e16x8 ov = *reinterpret_cast<const e16x8 *>(reinterpret_cast<const e16_t *>(a.o.ptr) +
-                                                          b * a.o.sb + (int64_t)i * a.o.ss + h * a.o.sh + 8 * c);
-      const e16x8 gv = *reinterpret_cast<const e16x8 *>(reinterpret_cast<const e16_t *>(a.d_o.ptr) +
-                                                          b * a.d_o.sb + (int64_t)i * a.d_o.ss +
-                                                          h * a.d_o.sh + 8 * c);
+  uint32_t b[kPrepRows], h[kPrepRows], i[kPrepRows];
+  bool real[kPrepRows];
+  e16x8 ov[kPrepRows], gv[kPrepRows];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc += (float)ov[e] * (float)gv[e];
+  for (int k = 0; k < kPrepRows; ++k) {
+    const uint32_t row = row0 + k * RPB;
+    if (hfast) {
+      const uint32_t t = row / H;
+      h[k] = row - t * H;
+      b[k] = t / Sqp;
+      i[k] = t - b[k] * Sqp;
+    } else {
+      const uint32_t t = row / Sqp;
+      i[k] = row - t * Sqp;
+      b[k] = t / H;
+      h[k] = t - b[k] * H;
+    }
+    real[k] = row < total && i[k] < (uint32_t)a.Sq;
+    ov[k] = gv[k] = e16x8{};
+    if (real[k]) {
+      ov[k] = *reinterpret_cast<const e16x8 *>(reinterpret_cast<const e16_t *>(a.o.ptr) + b[k] * a.o.sb +
+                                               (int64_t)i[k] * a.o.ss + h[k] * a.o.sh + 8 * c);
+      gv[k] = *reinterpret_cast<const e16x8 *>(reinterpret_cast<const e16_t *>(a.d_o.ptr) + b[k] * a.d_o.sb +
+                                               (int64_t)i[k] * a.d_o.ss + h[k] * a.d_o.sh + 8 * c);
     }
   }
 #pragma unroll
-  for (int o = LPR / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
-  if (row < total && c == 0) {
-    const bool ok = real && a.q_valid[(int64_t)b * a.Sq + i] != 0;
-    a.delta[row] = ok ? -acc : 0.f;  // stored negated: the dK/dV pairs start their dP accumulators from it
-    a.lse2[row] = ok ? a.lse[((int64_t)b * a.H + h) * a.Sq + i] * kLog2e : INFINITY;
+  for (int k = 0; k < kPrepRows; ++k) {
+    float acc = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc += (float)ov[k][e] * (float)gv[k][e];
+#pragma unroll
+    for (int o = LPR / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+    if (row0 + k * RPB < total && c == 0) {
+      const bool ok = real[k] && a.q_valid[(int64_t)b[k] * a.Sq + i[k]] != 0;
+      const int64_t out = ((int64_t)b[k] * H + h[k]) * Sqp + i[k];
+      a.delta[out] = ok ? -acc : 0.f;  // stored negated: the dK/dV pairs start their dP accumulators from it
+      a.lse2[out] = ok ? a.lse[((int64_t)b[k] * H + h[k]) * a.Sq + i[k]] * kLog2e : INFINITY;
+    }
   }
 }
 
@@ -1322,8 +1342,9 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
   if (!allow_dynamic_lds<&bwd_dq_kernel<D, NWQ>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
   if (!needed_table_fits(dq_smem_bytes<D>(), (a.Sk + 63) / 64)) return BCATTN_ERR_UNSUPPORTED;
   if (a.stages & BCATTN_BWD_DELTA) {
-    constexpr int RPB = 256 / (D / 8);
+    constexpr int RPB = 256 / (D / 8) * kPrepRows;
     const int64_t rows = (int64_t)a.B * a.H * a.Sq_pad;
+    if (rows >= (int64_t)1 << 31) return BCATTN_ERR_UNSUPPORTED;  // (32-bit row arithmetic in the kernel)
     hipLaunchKernelGGL(bwd_prep_kernel<D>, dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, st, a);
   }
   const int R = a.G * a.Sq;
