@@ -212,9 +212,8 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
   // from one phase into the next; every step (one product, its read, its share of the arithmetic) is
   // closed by pin_step(), the products and the arithmetic are tied to their step by empty asm
   // statements (without them instruction selection sinks them behind the last product).
-  // The running reference follows the half's maximum only when that has outgrown it by 2^8; O and the
-  // row sum are then rescaled between two phases (O is being accumulated into during the phase in
-  // which the second half's maximum is found).
+  // A half whose row sums show that the reference no longer fits is redone between two phases (O is
+  // being accumulated into during the phase that holds the second half's softmax).
   auto compute_il = [&](auto stage_c, auto masked_c, auto bg) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_c)::value != 0;
     constexpr int S = decltype(stage_c)::value;
@@ -245,9 +244,13 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
       if constexpr (nx < 2 * NPV) tv[nx % KC] = tra.template read<Vt>(nx / DB, nx % DB);
     };
     // ---- the softmax of one half, in the pieces that the steps of a phase take --------------
-    float mloc = 0.f, lt = 0.f, corr = 1.f, sv[16];  // sv: the half's scores, then its exponentials
+    // As at the smaller head dims, the exponentials are taken against the reference the row already has and
+    // the half's share of the row sum is the check (at most 2^13: no P left the range of the 16-bit types
+    // and of the fp32 sums).  Only when a row's sum is larger or not a number, or a valid row has no
+    // reference yet, is the half redone between two phases with the maxima found (redo_half).
+    constexpr float kSumMax = 8192.f;
+    float lt = 0.f, sv[16];  // sv: the half's scores, then its exponentials
     i32x4 kb4[4];
-    bool grown = false;
     // piece J of half H (J = 0 .. 15)
     auto softmax_piece = [&](auto h_c, auto j_c) __attribute__((always_inline)) {
       constexpr int H = decltype(h_c)::value, J = decltype(j_c)::value;
@@ -256,54 +259,74 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
 #pragma unroll
           for (int r4 = 0; r4 < 4; ++r4) kb4[r4] = *reinterpret_cast<const i32x4 *>(kb_s + 32 * H + 8 * r4 + 4 * hh);
         }
-      } else if constexpr (J <= 4) {  // out of the accumulator: mask and maximum of elements 4 (J-1) .. +3
+        lt = 0.f;
+      } else if constexpr (J <= 4) {  // out of the accumulator (and masked): elements 4 (J-1) .. +3
         constexpr int r4 = J - 1;
 #pragma unroll
         for (int x = 0; x < 4; ++x) {
           const int e = 4 * r4 + x;
           sv[e] = (MASKED && kb4[r4][x] > qb) ? -INFINITY : s[H][e];
-          mloc = e == 0 ? sv[0] : fmaxf(mloc, sv[e]);
         }
-        asm volatile("" : "+v"(mloc), "+v"(sv[4 * r4]), "+v"(sv[4 * r4 + 1]), "+v"(sv[4 * r4 + 2]), "+v"(sv[4 * r4 + 3]));
-      } else if constexpr (J == 5) {  // the row's maximum over the half; does the reference move?
-        mloc = fmaxf(mloc, swap32(mloc));
-        const bool grow = (mloc - m) * c > 8.f;  // false for a fully masked half (mloc = -inf)
-        const float mnew = grow ? mloc : m;
-        const float moff_new = (mnew == -INFINITY) ? 0.f : mnew * c;
-        // 1 where the reference stays; a row without one has accumulated nothing that counts
-        corr = !grow ? 1.f : (m == -INFINITY) ? 0.f : fast_exp2(moff - moff_new);
-        grown = __any(grow);
-        m = mnew;
-        moff = moff_new;
-        lt = 0.f;
-        asm volatile("" : "+v"(corr), "+v"(moff), "+v"(m));
-      } else if constexpr (J <= 13) {  // two exponentials
-        constexpr int e = 2 * (J - 6);
+        asm volatile("" : "+v"(sv[4 * r4]), "+v"(sv[4 * r4 + 1]), "+v"(sv[4 * r4 + 2]), "+v"(sv[4 * r4 + 3]));
+      } else if constexpr (J <= 12) {  // two exponentials
+        constexpr int e = 2 * (J - 5);
         sv[e] = fast_exp2(sv[e] * c - moff);
         sv[e + 1] = fast_exp2(sv[e + 1] * c - moff);
         lt += sv[e] + sv[e + 1];
         asm volatile("" : "+v"(sv[e]), "+v"(sv[e + 1]), "+v"(lt));
-      } else {  // eight of them to 16 bits
-        constexpr int q = J - 14;
+      } else if constexpr (J <= 14) {  // eight of them to 16 bits
+        constexpr int q = J - 13;
         pb[2 * H + q] = pack8(sv[8 * q], sv[8 * q + 1], sv[8 * q + 2], sv[8 * q + 3], sv[8 * q + 4], sv[8 * q + 5],
                               sv[8 * q + 6], sv[8 * q + 7]);
         asm volatile("" : "+v"(pb[2 * H + q]));
       }
     };
-    auto rescale = [&]() __attribute__((always_inline)) {
-      if (grown) {
-        // (O lives in accumulation registers; it is tied to them on both sides of this rare block, or the
-        // compiler keeps it in vector registers around the block and moves all of it on every tile)
+    // The half again, with its maxima: the reference follows a maximum that has outgrown it by 2^8, O and
+    // the row sum are rescaled (nothing accumulates into O between two phases), the exponentials are retaken.
+    auto redo_half = [&](auto h_c) __attribute__((always_inline)) {
+      constexpr int H = decltype(h_c)::value;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) asm volatile("" : "+a"(o[db]));
+      for (int db = 0; db < DB; ++db) asm volatile("" : "+a"(o[db]));
+      float mloc = -INFINITY;
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        i32x4 k4 = {0, 0, 0, 0};
+        if (MASKED) k4 = *reinterpret_cast<const i32x4 *>(kb_s + 32 * H + 8 * r4 + 4 * hh);
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          sv[4 * r4 + x] = (MASKED && k4[x] > qb) ? -INFINITY : s[H][4 * r4 + x];
+          mloc = fmaxf(mloc, sv[4 * r4 + x]);
+        }
+      }
+      mloc = fmaxf(mloc, swap32(mloc));
+      const bool grow = (mloc - m) * c > 8.f;  // false for a fully masked half (mloc = -inf)
+      const float mnew = grow ? mloc : m;
+      const float moff_new = (mnew == -INFINITY) ? 0.f : mnew * c;
+      if (__any(grow)) {
+        // 1 where the reference stays; a row without one has accumulated nothing that counts
+        const float corr = (m == -INFINITY) ? 0.f : fast_exp2(moff - moff_new);
         l *= corr;
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
           for (int x = 0; x < 16; ++x) o[db][x] *= corr;
-#pragma unroll
-        for (int db = 0; db < DB; ++db) asm volatile("" : "+a"(o[db]));
       }
+      m = mnew;
+      moff = moff_new;
+      lt = 0.f;
+#pragma unroll
+      for (int x = 0; x < 16; ++x) {
+        sv[x] = fast_exp2(sv[x] * c - moff);
+        lt += sv[x];
+      }
+      pb[2 * H] = pack8(sv[0], sv[1], sv[2], sv[3], sv[4], sv[5], sv[6], sv[7]);
+      pb[2 * H + 1] = pack8(sv[8], sv[9], sv[10], sv[11], sv[12], sv[13], sv[14], sv[15]);
+#pragma unroll
+      for (int db = 0; db < DB; ++db) asm volatile("" : "+a"(o[db]));
+    };
+    auto close_half = [&](auto h_c) __attribute__((always_inline)) {
+      const bool again = qv && (!(lt <= kSumMax) || m == -INFINITY);
+      if (__any(again)) redo_half(h_c);
       l += lt;
     };
     // ---- A: S of keys 0..31 ------------------------------------------------------------------
@@ -325,7 +348,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
       softmax_piece(StageC<0>{}, ks_c);
       pin_step();
     });
-    rescale();  // (P V of the tile before has long been issued; nothing accumulates into O in phase B)
+    close_half(StageC<0>{});  // (P V of the tile before has long been issued; nothing accumulates into O in phase B)
     pin_step();
     // ---- C: P V of half 0 beside the softmax of half 1 -----------------------------------------
     static_for<NPV>([&](auto i_c) {
@@ -336,7 +359,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
       softmax_piece(StageC<1>{}, i_c);
       pin_step();
     });
-    rescale();
+    close_half(StageC<1>{});
     pin_step();
     // ---- D: P V of half 1 ------------------------------------------------------------------------
     static_for<NPV>([&](auto i_c) {
