@@ -36,6 +36,12 @@ struct SplitStages {
 #ifndef BCATTN_FWD_INTERLEAVED
 #define BCATTN_FWD_INTERLEAVED 1
 #endif
+// Smallest head dim that takes the hand-ordered tile body (compute_il).  It is written for any head dim;
+// at head_dim 128, where two waves share a SIMD and cover each other's arithmetic, it measured 5 % slower
+// than the form that leaves the order inside a tile to the compiler.
+#ifndef BCATTN_FWD_INTERLEAVED_MIN_D
+#define BCATTN_FWD_INTERLEAVED_MIN_D 256
+#endif
 
 template <int D, int NW, bool SPLIT, bool TWOSEG>
 __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, const SplitArgs sp) {
@@ -221,6 +227,16 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
     const int *kb_s = reinterpret_cast<const int *>(smem + L::aux(S));
     constexpr int KA = 3, KC = 4;
     constexpr int NPV = 2 * DB;  // P V products of a half: (16-key quarter, 32-row block of O^T)
+    constexpr int PPS = 16 / DK;  // pieces of the softmax per step of a shared phase
+    static_assert(NPV == DK && PPS * DK == 16 && DK >= KC, "the shared phases have DK steps each");
+    // ties a product to its step: an empty asm statement over its accumulator, in the register file the
+    // accumulators of this kernel live in (accumulation registers where a wave has all 512, else vector)
+    auto tie = [](f32x16 &acc) __attribute__((always_inline)) {
+      if constexpr (D == 256)
+        asm volatile("" : "+a"(acc));
+      else
+        asm volatile("" : "+v"(acc));
+    };
     f32x16 s[2];
 #pragma unroll
     for (int mb = 0; mb < 2; ++mb)
@@ -286,7 +302,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
     auto redo_half = [&](auto h_c) __attribute__((always_inline)) {
       constexpr int H = decltype(h_c)::value;
 #pragma unroll
-      for (int db = 0; db < DB; ++db) asm volatile("" : "+a"(o[db]));
+      for (int db = 0; db < DB; ++db) tie(o[db]);
       float mloc = -INFINITY;
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
@@ -322,7 +338,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
       pb[2 * H] = pack8(sv[0], sv[1], sv[2], sv[3], sv[4], sv[5], sv[6], sv[7]);
       pb[2 * H + 1] = pack8(sv[8], sv[9], sv[10], sv[11], sv[12], sv[13], sv[14], sv[15]);
 #pragma unroll
-      for (int db = 0; db < DB; ++db) asm volatile("" : "+a"(o[db]));
+      for (int db = 0; db < DB; ++db) tie(o[db]);
     };
     auto close_half = [&](auto h_c) __attribute__((always_inline)) {
       const bool again = qv && (!(lt <= kSumMax) || m == -INFINITY);
@@ -334,7 +350,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
       constexpr int ks = decltype(ks_c)::value;
       parts_at_slot<ks, DK, LPT>(bg);  // (all requests in this phase: no vector arithmetic competes for issue)
       s[0] = mfma32(fk[ks % KA], qf[ks], s[0]);
-      asm volatile("" : "+a"(s[0]));
+      tie(s[0]);
       next_rows(StageC<ks + KA>{});
       pin_step();
     });
@@ -342,10 +358,10 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
     static_for<DK>([&](auto ks_c) {
       constexpr int ks = decltype(ks_c)::value;
       s[1] = mfma32(fk[(DK + ks) % KA], qf[ks], s[1]);
-      asm volatile("" : "+a"(s[1]));
+      tie(s[1]);
       next_rows(StageC<DK + ks + KA>{});
       if constexpr (ks >= DK - KC) next_cols(StageC<ks - (DK - KC)>{});
-      softmax_piece(StageC<0>{}, ks_c);
+      static_for<PPS>([&](auto pp) { softmax_piece(StageC<0>{}, StageC<ks * PPS + decltype(pp)::value>{}); });
       pin_step();
     });
     close_half(StageC<0>{});  // (P V of the tile before has long been issued; nothing accumulates into O in phase B)
@@ -354,9 +370,9 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
     static_for<NPV>([&](auto i_c) {
       constexpr int i = decltype(i_c)::value;
       o[i % DB] = mfma32(tv[i % KC], pb[i / DB], o[i % DB]);
-      asm volatile("" : "+a"(o[i % DB]));
+      tie(o[i % DB]);
       next_cols(StageC<i + KC>{});
-      softmax_piece(StageC<1>{}, i_c);
+      static_for<PPS>([&](auto pp) { softmax_piece(StageC<1>{}, StageC<i * PPS + decltype(pp)::value>{}); });
       pin_step();
     });
     close_half(StageC<1>{});
@@ -365,7 +381,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
     static_for<NPV>([&](auto i_c) {
       constexpr int i = NPV + decltype(i_c)::value;
       o[i % DB] = mfma32(tv[i % KC], pb[i / DB], o[i % DB]);
-      asm volatile("" : "+a"(o[i % DB]));
+      tie(o[i % DB]);
       next_cols(StageC<i + KC>{});
       pin_step();
     });
@@ -373,8 +389,7 @@ __global__ __launch_bounds__(64 * NW) void fwd_mfma_kernel(const FwdArgs a, cons
 
   auto compute_sm = [&](auto stage_c, const tile_summary_t sm, auto bg) __attribute__((always_inline)) {
     if (sm.x > qmax_w) return false;  // wave-uniform: no row of this wave sees a key of the tile
-    if constexpr (BCATTN_FWD_INTERLEAVED && D == 256) {
-      static_assert(DK == 2 * DB && DK == 16, "the phases are written for 16 steps each");
+    if constexpr (BCATTN_FWD_INTERLEAVED && D >= BCATTN_FWD_INTERLEAVED_MIN_D) {
       if (!(sm.z != 0 && sm.y <= qmin_w))
         compute_il(stage_c, StageC<1>{}, bg);
       else  // every row of the wave sees every key of the tile
