@@ -25,6 +25,10 @@
 
 #include "bcattn_tiles.h"
 
+#ifndef BCATTN_DQ_INTERLEAVED
+#define BCATTN_DQ_INTERLEAVED 1
+#endif
+
 namespace bcattn {
 inline namespace BCATTN_ELEM_NS {
 
@@ -283,13 +287,122 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a, const unsigned blo
       });
     });
   };
+  // head_dim 256 (one wave per SIMD: only the wave's own products can run beside its softmax / dS
+  // arithmetic): the tile in four phases of DK steps, as in the forward kernel of that head dim.
+  //   A: S and dP of keys 0..31 (with the tile requests)   B: S and dP of keys 32..63 beside the arithmetic of half 0
+  //   C: the dQ products of half 0 beside the arithmetic of half 1   D: the dQ products of half 1
+  // The row rings run on from A into B, the transposing ring from B (its last steps) through C and D.
+  auto compute_il = [&](auto stage_c, auto masked_c, auto bg) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_c)::value != 0;
+    constexpr int S = decltype(stage_c)::value;
+    constexpr int Kt = L::tile(S, 0), Vt = L::tile(S, 1);
+    const int *kb_s = reinterpret_cast<const int *>(smem + L::aux(S));
+    constexpr int KA = 3, KC = 4, NCS = 2 * DB;
+    static_assert(NCS == DK && DK == 16, "one element of a half's arithmetic per step");
+    f32x16 s[2], dp[2];
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) {
+      dp[mb] = nd16;  // dP starts from -delta of the lane's query: dS = P o dP' needs no subtraction
+#pragma unroll
+      for (int x = 0; x < 16; ++x) s[mb][x] = 0.f;
+    }
+    e16x8 fa[KA], fb[KA], ta[KC];
+    i32x4 wds[2][2], kb4[4];
+#pragma unroll
+    for (int i = 0; i < KA; ++i) {
+      fa[i] = rowa.template read<Kt>(0, i);
+      fb[i] = rowa.template read<Vt>(0, i);
+    }
+    pin_step();
+    auto next_rows = [&](auto nx_c) __attribute__((always_inline)) {
+      constexpr int nx = decltype(nx_c)::value;
+      if constexpr (nx < 2 * DK) {
+        fa[nx % KA] = rowa.template read<Kt>(32 * (nx / DK), nx % DK);
+        fb[nx % KA] = rowa.template read<Vt>(32 * (nx / DK), nx % DK);
+      }
+    };
+    auto next_cols = [&](auto nx_c) __attribute__((always_inline)) {
+      constexpr int nx = decltype(nx_c)::value;
+      if constexpr (nx < 2 * NCS) ta[nx % KC] = tra.template read<Kt>(nx / DB, nx % DB);
+    };
+    // element J of half H: P = exp2(c S - log2e LSE) (masked), dS = P o dP'; every second step packs a pair
+    float dsf = 0.f;
+    auto ds_piece = [&](auto h_c, auto j_c) __attribute__((always_inline)) {
+      constexpr int H = decltype(h_c)::value, J = decltype(j_c)::value;
+      if constexpr (MASKED && J == 0) {
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) kb4[r4] = *reinterpret_cast<const i32x4 *>(kb_s + 32 * H + 8 * r4 + 4 * hh);
+      }
+      float p = fast_exp2(s[H][J] * c - lse2);
+      if (MASKED && kb4[J / 4][J % 4] > qb) p = 0.f;
+      const float d = p * dp[H][J];
+      if constexpr (J % 2 == 0) {
+        dsf = d;
+        asm volatile("" : "+v"(dsf));
+      } else {
+        typedef e16_t e16x2_t __attribute__((ext_vector_type(2)));
+        e16x2_t r;
+        r[0] = (e16_t)dsf;
+        r[1] = (e16_t)d;
+        wds[H][J / 8][(J % 8) / 2] = __builtin_bit_cast(int, r);
+        asm volatile("" : "+v"(wds[H][J / 8][(J % 8) / 2]));
+      }
+    };
+    static_for<DK>([&](auto ks_c) {  // ---- A
+      constexpr int ks = decltype(ks_c)::value;
+      parts_at_slot<ks, DK, LPT>(bg);
+      s[0] = mfma32(fa[ks % KA], qf[ks], s[0]);
+      dp[0] = mfma32(fb[ks % KA], gof[ks], dp[0]);
+      asm volatile("" : "+a"(s[0]), "+a"(dp[0]));
+      next_rows(StageC<ks + KA>{});
+      pin_step();
+    });
+    static_for<DK>([&](auto ks_c) {  // ---- B
+      constexpr int ks = decltype(ks_c)::value;
+      s[1] = mfma32(fa[(DK + ks) % KA], qf[ks], s[1]);
+      dp[1] = mfma32(fb[(DK + ks) % KA], gof[ks], dp[1]);
+      asm volatile("" : "+a"(s[1]), "+a"(dp[1]));
+      next_rows(StageC<DK + ks + KA>{});
+      if constexpr (ks >= DK - KC) next_cols(StageC<ks - (DK - KC)>{});
+      ds_piece(StageC<0>{}, ks_c);
+      pin_step();
+    });
+    e16x8 dsb[4];
+    dsb[0] = __builtin_bit_cast(e16x8, wds[0][0]);
+    dsb[1] = __builtin_bit_cast(e16x8, wds[0][1]);
+    static_for<NCS>([&](auto i_c) {  // ---- C
+      constexpr int i = decltype(i_c)::value;
+      dq[i % DB] = mfma32(ta[i % KC], dsb[i / DB], dq[i % DB]);
+      asm volatile("" : "+a"(dq[i % DB]));
+      next_cols(StageC<i + KC>{});
+      ds_piece(StageC<1>{}, i_c);
+      pin_step();
+    });
+    dsb[2] = __builtin_bit_cast(e16x8, wds[1][0]);
+    dsb[3] = __builtin_bit_cast(e16x8, wds[1][1]);
+    static_for<NCS>([&](auto i_c) {  // ---- D
+      constexpr int i = NCS + decltype(i_c)::value;
+      dq[i % DB] = mfma32(ta[i % KC], dsb[i / DB], dq[i % DB]);
+      asm volatile("" : "+a"(dq[i % DB]));
+      next_cols(StageC<i + KC>{});
+      pin_step();
+    });
+  };
   auto compute = [&](auto stage_c, const i32x4 e, auto bg) __attribute__((always_inline)) {
     const tile_summary_t sm = {e.y, e.z, e.w, 0};
     if (sm.x > qmax_w) return false;  // wave-uniform: no row of this wave sees a key of the tile
-    if (sm.z != 0 && sm.y <= qmin_w)
-      compute_t(stage_c, StageC<0>{}, bg);  // every pair of the tile attends
-    else
-      compute_t(stage_c, StageC<1>{}, bg);
+    const bool masked = !(sm.z != 0 && sm.y <= qmin_w);  // false: every pair of the tile attends
+    if constexpr (BCATTN_DQ_INTERLEAVED && D == 256) {
+      if (masked)
+        compute_il(stage_c, StageC<1>{}, bg);
+      else
+        compute_il(stage_c, StageC<0>{}, bg);
+    } else {
+      if (masked)
+        compute_t(stage_c, StageC<1>{}, bg);
+      else
+        compute_t(stage_c, StageC<0>{}, bg);
+    }
     return true;
   };
 
