@@ -85,3 +85,55 @@ def test_cache_rejects_rows_that_do_not_fit():
         cache.fill(0, k, k)
     with pytest.raises(RuntimeError, match="fit"):
         cache.fill(0, k[:1, :4], k[:1, :4])
+
+
+def test_whole_denoise_loop_replays_from_one_graph():
+    """The pi0.5 inference loop at its real depth, 10 flow-matching steps x 18 layers of [rotate q and k ;
+    attend over the cached prefix and the step's own keys] through the static cache
+    (``pi05/modeling_pi05.py:2015-2046``, ``paligemma_with_expert.py:742-768``), captured as ONE HIP graph:
+    every replay, on new inputs in the captured buffers and with eager work in between, gives bit for bit
+    what the same loop gives when called eagerly (the mask's summary is made once, before the capture; the
+    calls allocate through the graph's pool only and clear nothing)."""
+    layers, steps, b, n_pre, n_act, h, hkv, d = 18, 10, 2, 200, 50, 8, 1, 256
+    dt = torch.bfloat16
+    pre_pad = torch.ones(b, n_pre, dtype=torch.bool)
+    pre_pad[1, -13:] = False
+    pre_pos = (torch.cumsum(pre_pad, 1) - 1).clamp_min(0)
+    cache = StaticKVCache(layers, b, 256, hkv, d, dt, DEV)
+    for layer in range(layers):
+        cache.fill(layer, g(randn((b, n_pre, hkv, d), dt, 3 * layer)), g(randn((b, n_pre, hkv, d), dt, 3 * layer + 1)),
+                   positions=g(pre_pos))
+    suf_pad = torch.ones(b, n_act, dtype=torch.bool)
+    suf_att = torch.zeros(b, n_act, dtype=torch.int32)
+    suf_att[:, 0] = 1
+    ids = tuple(g(t) for t in fa.make_att_block_ids(suf_pad, suf_att, n_pre, pre_pad))
+    suf_pos = g(pre_pad.sum(1, keepdim=True) + torch.arange(n_act)[None])
+    qs = g(randn((layers, b, n_act, h, d), dt, 500))
+    ks, vs = g(randn((layers, b, n_act, hkv, d), dt, 501)), g(randn((layers, b, n_act, hkv, d), dt, 502))
+
+    def loop():
+        outs = []
+        for step in range(steps):
+            gain = 1.0 + 0.03 * step  # (a step's inputs differ from the last step's)
+            for layer in range(layers):
+                q, k = apply_rope_qk(qs[layer] * gain, ks[layer], suf_pos)
+                outs.append(cache.attend(layer, q, k, vs[layer], ids))
+        return outs
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):  # first calls outside the capture: kernel attributes, the mask's summary
+        loop()
+    side.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = loop()
+    assert len(captured) == steps * layers
+    for rep in range(3):
+        for t, seed in ((qs, 600), (ks, 601), (vs, 602)):
+            t.copy_(g(randn(tuple(t.shape), dt, seed + 10 * rep)))
+        graph.replay()
+        torch.cuda.synchronize()
+        eager_outs = loop()
+        torch.cuda.synchronize()
+        assert all(torch.equal(a, e) for a, e in zip(captured, eager_outs)), rep
+        assert float(captured[-1].float().abs().sum()) > 0
