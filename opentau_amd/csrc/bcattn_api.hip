@@ -243,7 +243,7 @@ size_t bcattn_bwd_workspace_bytes(const bcattn_bwd_params *p) {
   if (p == nullptr || p->B <= 0) return 0;
   return summary_bytes(p->B, p->Sk, p->Sk) + merged_bytes(p->B, p->Sk, p->Sk) +
          summary_bytes(p->B, p->Sq, p->Sq) + merged_bytes(p->B, p->Sq, p->Sq) +
-         2 * align256((size_t)p->B * p->H * pad64(p->Sq) * sizeof(float)) +
+         2 * align256((size_t)p->B * p->H * pad64(p->Sq) * sizeof(float)) + kBwdQueueBytes +
          (p->Hkv > 0 ? bwd_dkv_part_bytes(p->B, p->Sq, p->Sk, p->Hkv, p->H / p->Hkv, p->D, p->dtype) : 0);
 }
 
@@ -359,7 +359,8 @@ int bcattn_bwd(const bcattn_bwd_params *p, void *stream) {
   a.scale = p->scale;
   a.stages = p->stages & (BCATTN_BWD_DELTA | BCATTN_BWD_DQ | BCATTN_BWD_DKV);
   if (a.stages == 0) a.stages = BCATTN_BWD_DELTA | BCATTN_BWD_DQ | BCATTN_BWD_DKV;
-  // Backward workspace: [key summaries][key ids][query summaries][query ids][delta][log2e*LSE][dK/dV partial sums].
+  // Backward workspace: [key summaries][key ids][query summaries][query ids][delta][log2e*LSE][work counters]
+  // [dK/dV partial sums].
   char *ws = reinterpret_cast<char *>(p->workspace);
   tile_summary_t *ks = reinterpret_cast<tile_summary_t *>(ws);
   ws += summary_bytes(a.B, a.Sk, a.Sk);
@@ -373,6 +374,8 @@ int bcattn_bwd(const bcattn_bwd_params *p, void *stream) {
   ws += align256((size_t)a.B * a.H * a.Sq_pad * sizeof(float));
   a.lse2 = reinterpret_cast<float *>(ws);
   ws += align256((size_t)a.B * a.H * a.Sq_pad * sizeof(float));
+  a.queue = reinterpret_cast<unsigned *>(ws);
+  ws += kBwdQueueBytes;
   a.dkv_splits = bwd_dkv_splits(a.B, a.Sq, a.Sk, a.Hkv, a.G, p->D, p->dtype);
   a.dkv_part = reinterpret_cast<float *>(ws);
   a.ksum = ks, a.qsum = qs, a.kbm = km, a.qbm = qm;

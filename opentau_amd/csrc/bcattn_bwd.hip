@@ -32,6 +32,15 @@
 namespace bcattn {
 inline namespace BCATTN_ELEM_NS {
 
+// The thread's index in its workgroup, made opaque to the compiler once per work item: a kernel that
+// loops over work items of several kinds would otherwise keep every lane-dependent address and offset
+// of every kind of item in registers for the whole loop (they are loop-invariant to it).
+__device__ __forceinline__ int item_local_tid() {
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));
+  return tid;
+}
+
 // ---- prep: delta and scaled LSE, padded -------------------------------------------
 // One row (b, h, i) per D/8 lanes, kPrepRows rows per thread with all of their loads in flight
 // together.  Rows are taken in the order in which they lie in memory: heads fastest where a token's
@@ -44,6 +53,7 @@ __global__ __launch_bounds__(256) void bwd_prep_kernel(const BwdArgs a) {
   const uint32_t Sqp = (uint32_t)a.Sq_pad, H = (uint32_t)a.H;
   const uint32_t total = (uint32_t)a.B * H * Sqp;  // (the launcher checks that this fits)
   const bool hfast = a.o.sh < a.o.ss;
+  if (blockIdx.x == 0 && threadIdx.x < kXcds) a.queue[threadIdx.x] = 0;  // the work counters of the launch behind this one
   const uint32_t row0 = blockIdx.x * (uint32_t)(RPB * kPrepRows) + threadIdx.x / LPR;
   const int c = threadIdx.x % LPR;
   uint32_t b[kPrepRows], h[kPrepRows], i[kPrepRows];
@@ -107,7 +117,7 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a, const unsigned blo
   extern __shared__ __align__(1024) char smem[];
   __shared__ int red_s[2 * NW];
 
-  const int tid = threadIdx.x;
+  const int tid = item_local_tid();
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
 
@@ -450,7 +460,7 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, const unsigned bl
   extern __shared__ __align__(1024) char smem[];
   __shared__ int red_s[NW];
 
-  const int tid = threadIdx.x;
+  const int tid = item_local_tid();
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
 
@@ -899,7 +909,7 @@ __device__ __forceinline__ void bwd_dkv_pair_body(const BwdArgs &a, const unsign
   extern __shared__ __align__(1024) char smem[];
   __shared__ int red_s[NP];
 
-  const int tid = threadIdx.x;
+  const int tid = item_local_tid();
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int n = lane & 31, hh = lane >> 5;
   const bool pwave = wave < NP;  // wave-uniform role
@@ -1367,40 +1377,105 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
 // dK/dV and dQ in one launch.  The two are independent, and each alone leaves part of the chip idle
 // while its last workgroups finish (a workgroup holds most of a CU's LDS, so a grid is a small number
 // of "rounds" of one workgroup per CU, and a dK/dV workgroup runs several times as long as a dQ
-// workgroup).  Workgroups are handed out in index order: the dK/dV workgroups take the first
-// indices, so all of the long ones start first and the short dQ workgroups fill the CUs as they
-// come free, up to the very end.  (Every role's share of the grid is a multiple of 8 workgroups, so
-// each keeps its own XCD mapping.)
-template <int D, int NWQ, int NP>
-__global__ __launch_bounds__(128 * NP) void bwd_dkv_dq_kernel(const BwdArgs a, const unsigned ndkv) {
-  static_assert(64 * NWQ == 128 * NP, "both roles use the same workgroup size");
-  warm_kernel_arguments<sizeof(BwdArgs) + sizeof(unsigned)>();
-  if (blockIdx.x < ndkv)
-    bwd_dkv_pair_body<D, NP>(a, blockIdx.x);
-  else
-    bwd_dq_body<D, NWQ>(a, blockIdx.x - ndkv);
+// workgroup).  The launch has as many workgroups as the chip holds at once, and each draws work items
+// until none is left: the dK/dV items come first, so all of the long ones start first and the short dQ
+// items fill the CUs as they come free, up to the very end.  (Left to the hardware's dispatcher, which
+// hands out the workgroups of a grid in index order, a CU whose workgroup finished early stayed idle
+// while later workgroups waited: 10-15 % of the CUs at any time on the pi0.5 / pi0.6 training shapes.)
+// Items are numbered like the workgroups of a plain launch were, item % kXcds being the XCD that takes it
+// (every role's share is a multiple of kXcds), and XCD x draws its items in order from counter x, so
+// consecutive items, which stream the same Q/dO or K/V, still meet in one L2.  Nothing waits for
+// another workgroup: a workgroup leaves when its counter has run past the last item.  The results do
+// not depend on which workgroup computes an item.
+// An item is a call of a function of its own (not inlined): inlined into the loop, the lane-dependent
+// addresses and the arguments of every kind of item stay in registers across the whole loop and spill.
+__device__ __forceinline__ unsigned bwd_queue_next(unsigned *queue, unsigned *slot) {
+  const unsigned xcd = blockIdx.x % kXcds;
+  __syncthreads();  // every wave is done with the item before (its LDS, and its copy of the slot)
+  if (threadIdx.x == 0) *slot = atomicAdd(queue + xcd, 1u);
+  __syncthreads();
+  return __builtin_amdgcn_readfirstlane(*slot) * kXcds + xcd;
+}
+__global__ void bwd_queue_zero_kernel(unsigned *queue) {
+  if (threadIdx.x < kXcds) queue[threadIdx.x] = 0;
+}
+// The launch's first argument as the item functions read it: from the argument segment, by scalar loads.
+__device__ __forceinline__ BwdArgs first_kernel_argument() {
+#if defined(__HIP_DEVICE_COMPILE__)
+  typedef const __attribute__((address_space(4))) BwdArgs *args_ptr_t;
+  args_ptr_t p = (args_ptr_t)__builtin_amdgcn_kernarg_segment_ptr();
+  asm volatile("" : "+s"(p));  // (read again for every item: not carried in registers across the loop)
+  return *p;
+#else
+  return BwdArgs{};
+#endif
+}
+template <int D, int NP>
+__device__ __forceinline__ void bwd_dkv_pair_item(unsigned item) {
+  const BwdArgs a = first_kernel_argument();
+  bwd_dkv_pair_body<D, NP>(a, __builtin_amdgcn_readfirstlane(item));  // (arguments arrive in vector registers)
+}
+template <int D, int NW, int MODE>
+__device__ __forceinline__ void bwd_dkv_item(unsigned item) {
+  const BwdArgs a = first_kernel_argument();
+  bwd_dkv_body<D, NW, MODE>(a, __builtin_amdgcn_readfirstlane(item));  // (arguments arrive in vector registers)
+}
+template <int D, int NW>
+__device__ __forceinline__ void bwd_dq_item(unsigned item) {
+  const BwdArgs a = first_kernel_argument();
+  bwd_dq_body<D, NW>(a, __builtin_amdgcn_readfirstlane(item));  // (arguments arrive in vector registers)
 }
 
-// The same for the single-wave dK/dV forms.  TWO: dK/dV as two sets of `ndkv` workgroups (dV alone,
-// then dK alone: the form head_dim 256 takes).  (Measured on the pi0.5 / pi0.6 training shapes: with
-// the dK set in front of the dV set the step is 7 % slower; dQ workgroups placed between the two sets
-// change nothing.)
-template <int D, int NW, bool TWO>
-__global__ __launch_bounds__(64 * NW) void bwd_dkv1_dq_kernel(const BwdArgs a, const unsigned ndkv) {
-  warm_kernel_arguments<sizeof(BwdArgs) + sizeof(unsigned)>();
-  if constexpr (TWO) {
-    if (blockIdx.x < ndkv)
-      bwd_dkv_body<D, NW, kModeDV>(a, blockIdx.x);
-    else if (blockIdx.x < 2 * ndkv)
-      bwd_dkv_body<D, NW, kModeDK>(a, blockIdx.x - ndkv);
+template <int D, int NWQ, int NP>
+__global__ __launch_bounds__(128 * NP) void bwd_dkv_dq_kernel(const BwdArgs a, const unsigned ndkv, const unsigned nitems) {
+  static_assert(64 * NWQ == 128 * NP, "both roles use the same workgroup size");
+  warm_kernel_arguments<sizeof(BwdArgs) + 2 * sizeof(unsigned)>();
+  __shared__ unsigned slot;
+  for (;;) {
+    const unsigned item = bwd_queue_next(a.queue, &slot);
+    if (item >= nitems) break;
+    if (item < ndkv)
+      bwd_dkv_pair_item<D, NP>(item);
     else
-      bwd_dq_body<D, NW>(a, blockIdx.x - 2 * ndkv);
-  } else {
-    if (blockIdx.x < ndkv)
-      bwd_dkv_body<D, NW, kModeBoth>(a, blockIdx.x);
-    else
-      bwd_dq_body<D, NW>(a, blockIdx.x - ndkv);
+      bwd_dq_item<D, NWQ>(item - ndkv);
   }
+}
+
+// The same for the single-wave dK/dV forms.  TWO: dK/dV as two sets of `ndkv` items (dV alone,
+// then dK alone: the form head_dim 256 takes).
+template <int D, int NW, bool TWO>
+__global__ __launch_bounds__(64 * NW) void bwd_dkv1_dq_kernel(const BwdArgs a, const unsigned ndkv, const unsigned nitems) {
+  warm_kernel_arguments<sizeof(BwdArgs) + 2 * sizeof(unsigned)>();
+  __shared__ unsigned slot;
+  for (;;) {
+    const unsigned item = bwd_queue_next(a.queue, &slot);
+    if (item >= nitems) break;
+    if constexpr (TWO) {
+      if (item < ndkv)
+        bwd_dkv_item<D, NW, kModeDV>(item);
+      else if (item < 2 * ndkv)
+        bwd_dkv_item<D, NW, kModeDK>(item - ndkv);
+      else
+        bwd_dq_item<D, NW>(item - 2 * ndkv);
+    } else {
+      if (item < ndkv)
+        bwd_dkv_item<D, NW, kModeBoth>(item);
+      else
+        bwd_dq_item<D, NW>(item - ndkv);
+    }
+  }
+}
+
+// Workgroups of `kernel` that the chip holds at once (a multiple of kXcds, at least kXcds).
+template <class K>
+static unsigned resident_workgroups(K kernel, int threads, size_t smem) {
+  int per_cu = 0, dev = 0, cus = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, smem) != hipSuccess || per_cu < 1) per_cu = 1;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
+    cus = kXcds;
+  const unsigned n = (unsigned)per_cu * (unsigned)cus / kXcds * kXcds;
+  return n < kXcds ? kXcds : n;
 }
 
 template <int D, int NP>
@@ -1470,19 +1545,26 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
   const bool reduce = (a.stages & BCATTN_BWD_DKV) && a.dkv_splits > 1;
   const bool both = (a.stages & BCATTN_BWD_DQ) && (a.stages & BCATTN_BWD_DKV);
   if (both && !serial_backward()) {
+    // (the prep kernel, when it runs in this call, has zeroed the work counters)
+    if (!(a.stages & BCATTN_BWD_DELTA)) hipLaunchKernelGGL(bwd_queue_zero_kernel, dim3(1), dim3(64), 0, st, a.queue);
     if constexpr (PAIRS > 0) {
       if (!allow_dynamic_lds<&bwd_dkv_dq_kernel<D, NWQ, PAIRS>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
       if (!needed_table_fits(dkv_pair_smem_bytes<D, PAIRS>(), a.Sq_pad / 64)) return BCATTN_ERR_UNSUPPORTED;
       const size_t smem_kv = dkv_pair_smem_bytes<D, PAIRS>() + needed_table_bytes(a.Sq_pad / 64);
-      hipLaunchKernelGGL((bwd_dkv_dq_kernel<D, NWQ, PAIRS>), dim3(ndkv + ndq), dim3(128 * PAIRS),
-                         smem_kv > smem_q ? smem_kv : smem_q, st, a, ndkv);
+      const size_t smem = smem_kv > smem_q ? smem_kv : smem_q;
+      const unsigned nitems = ndkv + ndq, fit = resident_workgroups(bwd_dkv_dq_kernel<D, NWQ, PAIRS>, 128 * PAIRS, smem);
+      hipLaunchKernelGGL((bwd_dkv_dq_kernel<D, NWQ, PAIRS>), dim3(nitems < fit ? nitems : fit), dim3(128 * PAIRS), smem, st,
+                         a, ndkv, nitems);
     } else {
       static_assert(NWQ == NWK, "both roles use the same workgroup size");
       if (!allow_dynamic_lds<&bwd_dkv1_dq_kernel<D, NWQ, SPLIT>>((int)(kLdsBytes - 1024))) return BCATTN_ERR_LAUNCH;
       if (!needed_table_fits(dkv_smem_bytes<D>(), a.Sq_pad / 64)) return BCATTN_ERR_UNSUPPORTED;
       const size_t smem_kv = dkv_smem_bytes<D>() + needed_table_bytes(a.Sq_pad / 64);
-      hipLaunchKernelGGL((bwd_dkv1_dq_kernel<D, NWQ, SPLIT>), dim3((SPLIT ? 2 : 1) * ndkv + ndq), dim3(64 * NWQ),
-                         smem_kv > smem_q ? smem_kv : smem_q, st, a, ndkv);
+      const size_t smem = smem_kv > smem_q ? smem_kv : smem_q;
+      const unsigned nitems = (SPLIT ? 2 : 1) * ndkv + ndq,
+                     fit = resident_workgroups(bwd_dkv1_dq_kernel<D, NWQ, SPLIT>, 64 * NWQ, smem);
+      hipLaunchKernelGGL((bwd_dkv1_dq_kernel<D, NWQ, SPLIT>), dim3(nitems < fit ? nitems : fit), dim3(64 * NWQ), smem, st,
+                         a, ndkv, nitems);
     }
     if (reduce) launch_dkv_reduce<D>(a, st);
     return hipGetLastError() == hipSuccess ? BCATTN_OK : BCATTN_ERR_LAUNCH;

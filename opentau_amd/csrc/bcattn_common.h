@@ -173,7 +173,11 @@ struct BwdArgs {
   // ([dK | dV][split][B][Sk][Hkv][D]) that a second kernel adds in a fixed order.  1: no split.
   int dkv_splits;
   float *dkv_part;
+  // kXcds counters (zeroed on the stream before the launch that uses them): the workgroups of the
+  // backward's single launch draw their work items from them (see bwd_queue_next)
+  unsigned *queue;
 };
+constexpr size_t kBwdQueueBytes = 256;
 
 // How many workgroups share a key block's query heads in the 16-bit dK/dV kernels (a divisor of G).  The
 // kernels take 128 keys per workgroup; a launch of fewer than kDkvFill of them leaves most of the chip idle
