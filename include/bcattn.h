@@ -137,6 +137,10 @@ typedef struct bcattn_bwd_params {
   int32_t stages;
   /* Nonzero: the workspace already holds the tile summaries of these masks. */
   int32_t summary_ready;
+  /*
+   * Written by the call's kernels (delta, the work counters of the dQ + dK/dV launch,
+   * partial sums): calls that may run at the same time need a workspace each.
+   */
   void *workspace;
   size_t workspace_bytes;
 } bcattn_bwd_params;
