@@ -645,6 +645,35 @@ def test_dispatch_surface_matches_sdpa(pattern):
     assert_close_bf16(flash_out * vr, eager_out * vr, "out")
 
 
+def test_memory_reduction_vs_eager():
+    """The reference's headline guarantee (``tests/policies/test_flash_attn_cuda.py:380-442``): the fused call
+    never builds the S x S scores or the dense mask, so its peak memory stays far below the eager path's.  Same
+    shape as there (B2 S1024 H8 Hkv1 D256 bf16, prefix-LM); held here to a bound as well: the output, the
+    row statistics and the tile summaries, nothing that grows with S squared."""
+    b, s, h, hkv, d = 2, 1024, 8, 1, 256
+    q, k, v = (g(t) for t in _qkv(b, s, s, h, hkv, d, torch.bfloat16))
+    ids_cpu = make_blocks(b, s, "prefixlm")
+    ids = [g(t) for t in ids_cpu]
+    dense = g(eager.make_att_2d_masks(ids_cpu[2], att_masks("prefixlm", b, s)))
+
+    def peak(fn):
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        base = torch.cuda.memory_allocated()
+        out = fn()
+        torch.cuda.synchronize()
+        return (torch.cuda.max_memory_allocated() - base) / 1e6, out
+
+    flash_mem, flash_out = peak(lambda: fa.flash_attn_blockmask(q, k, v, *ids, d**-0.5))
+    eager_mem, eager_out = peak(lambda: eager.eager_attention_bshd(dense, q, k, v))
+    assert flash_mem < eager_mem
+    out_mb = flash_out.numel() * flash_out.element_size() / 1e6
+    scores_mb = b * h * s * s * 4 / 1e6
+    assert flash_mem <= out_mb + 1.0, f"peak {flash_mem:.2f} MB for an output of {out_mb:.2f} MB"
+    assert eager_mem >= scores_mb  # (what the fused call avoids)
+    assert_close_bf16(flash_out.reshape(b, s, h * d).float().cpu(), eager_out.float().cpu(), "out")
+
+
 def test_autograd_op_matches_raw_backward():
     b, sq, h, hkv, d = 2, 70, 4, 2, 128
     ids = [g(t) for t in make_blocks(b, sq, "multiblock", pad_tail=5)]
