@@ -1387,8 +1387,9 @@ __global__ __launch_bounds__(128 * NP) void bwd_dkv_pair_kernel(const BwdArgs a)
 // consecutive items, which stream the same Q/dO or K/V, still meet in one L2.  Nothing waits for
 // another workgroup: a workgroup leaves when its counter has run past the last item.  The results do
 // not depend on which workgroup computes an item.
-// An item is a call of a function of its own (not inlined): inlined into the loop, the lane-dependent
-// addresses and the arguments of every kind of item stay in registers across the whole loop and spill.
+// An item reads the launch's arguments again from the argument segment and takes the lane index through
+// an opaque copy (item_local_tid): written plainly, the lane-dependent addresses and the arguments of
+// every kind of item are hoisted out of the loop, stay in registers across all of it, and spill.
 __device__ __forceinline__ unsigned bwd_queue_next(unsigned *queue, unsigned *slot) {
   const unsigned xcd = blockIdx.x % kXcds;
   __syncthreads();  // every wave is done with the item before (its LDS, and its copy of the slot)
@@ -1466,16 +1467,24 @@ __global__ __launch_bounds__(64 * NW) void bwd_dkv1_dq_kernel(const BwdArgs a, c
   }
 }
 
-// Workgroups of `kernel` that the chip holds at once (a multiple of kXcds, at least kXcds).
-template <class K>
-static unsigned resident_workgroups(K kernel, int threads, size_t smem) {
-  int per_cu = 0, dev = 0, cus = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, smem) != hipSuccess || per_cu < 1) per_cu = 1;
-  if (hipGetDevice(&dev) != hipSuccess ||
-      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
-    cus = kXcds;
-  const unsigned n = (unsigned)per_cu * (unsigned)cus / kXcds * kXcds;
-  return n < kXcds ? kXcds : n;
+// Workgroups of `kernel` that the chip holds at once (a multiple of kXcds, at least kXcds).  The answer
+// for the last (device, LDS size) asked is kept per kernel: a training loop asks the same one every step.
+template <auto Kernel>
+static unsigned resident_workgroups(int threads, size_t smem) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+  // one word, so that threads asking at once read and write it whole: device (8 bits), LDS bytes (24), answer (32)
+  static std::atomic<uint64_t> last{0};
+  const uint64_t key = ((uint64_t)(dev & 0xff) << 56) | ((uint64_t)(smem & 0xffffff) << 32);
+  const uint64_t seen = last.load(std::memory_order_relaxed);
+  if ((seen >> 32) == (key >> 32) && (uint32_t)seen != 0) return (uint32_t)seen;
+  int per_cu = 0, cus = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, Kernel, threads, smem) != hipSuccess || per_cu < 1) per_cu = 1;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1) cus = kXcds;
+  unsigned n = (unsigned)per_cu * (unsigned)cus / kXcds * kXcds;
+  if (n < kXcds) n = kXcds;
+  last.store(key | n, std::memory_order_relaxed);
+  return n;
 }
 
 template <int D, int NP>
@@ -1552,7 +1561,7 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
       if (!needed_table_fits(dkv_pair_smem_bytes<D, PAIRS>(), a.Sq_pad / 64)) return BCATTN_ERR_UNSUPPORTED;
       const size_t smem_kv = dkv_pair_smem_bytes<D, PAIRS>() + needed_table_bytes(a.Sq_pad / 64);
       const size_t smem = smem_kv > smem_q ? smem_kv : smem_q;
-      const unsigned nitems = ndkv + ndq, fit = resident_workgroups(bwd_dkv_dq_kernel<D, NWQ, PAIRS>, 128 * PAIRS, smem);
+      const unsigned nitems = ndkv + ndq, fit = resident_workgroups<&bwd_dkv_dq_kernel<D, NWQ, PAIRS>>(128 * PAIRS, smem);
       hipLaunchKernelGGL((bwd_dkv_dq_kernel<D, NWQ, PAIRS>), dim3(nitems < fit ? nitems : fit), dim3(128 * PAIRS), smem, st,
                          a, ndkv, nitems);
     } else {
@@ -1562,7 +1571,7 @@ static int launch_bwd_d(const BwdArgs &a, hipStream_t st) {
       const size_t smem_kv = dkv_smem_bytes<D>() + needed_table_bytes(a.Sq_pad / 64);
       const size_t smem = smem_kv > smem_q ? smem_kv : smem_q;
       const unsigned nitems = (SPLIT ? 2 : 1) * ndkv + ndq,
-                     fit = resident_workgroups(bwd_dkv1_dq_kernel<D, NWQ, SPLIT>, 64 * NWQ, smem);
+                     fit = resident_workgroups<&bwd_dkv1_dq_kernel<D, NWQ, SPLIT>>(64 * NWQ, smem);
       hipLaunchKernelGGL((bwd_dkv1_dq_kernel<D, NWQ, SPLIT>), dim3(nitems < fit ? nitems : fit), dim3(64 * NWQ), smem, st,
                          a, ndkv, nitems);
     }
